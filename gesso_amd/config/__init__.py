@@ -1,5 +1,6 @@
 from .lfm2 import Lfm2Config, adjusted_ff_dim
+from .makuzen import LatentAttentionConfig, MakuzenConfig, MakuzenLayer, TableMoEConfig, YarnScaling
 from .registry import (architecture_of, load_config, register_architecture, registered_architectures,
                        unregister_architecture)
-from .spec import (AttentionSpec, BlockSpec, LayerCall, ModelSpec, NoPositionSpec, RMSNormSpec, RopeSpec,
-                   ShortConvSpec, SwiGLUSpec)
+from .spec import (AttentionSpec, BlockSpec, LatentAttentionSpec, LayerCall, ModelSpec, NoPositionSpec,
+                   OutNormBlockSpec, RMSNormSpec, RopeSpec, ScaledRopeSpec, ShortConvSpec, SwiGLUSpec, TableMoESpec)

@@ -1,7 +1,7 @@
 """One registry from an architecture's name to its configuration type and model factory.
 
-``config.json`` names the architecture in ``architectures[0]``; the entry registered under
-that name parses the file's keys into a typed configuration and turns the configuration
+``config.json`` names the architecture in ``architectures[0]`` or, as one string, under
+``architecture``; the entry registered under that name parses the file's keys into a typed configuration and turns the configuration
 into a :class:`~gesso_amd.config.spec.ModelSpec`.  The reference's counterpart is the
 adapter table ``_ADAPTERS`` with ``adapter_for`` (``src/Inference/arch_adapters.jl:1075-1109``),
 whose error lists the known names; so does ours.
@@ -44,8 +44,10 @@ def registered_architectures():
 
 def architecture_of(raw: dict) -> Architecture:
     names = raw.get("architectures")
+    if names is None and isinstance(raw.get("architecture"), str):
+        names = [raw["architecture"]]
     if not (isinstance(names, list) and len(names) >= 1 and isinstance(names[0], str)):
-        raise ConfigError("config.json must name its model in architectures[0]",
+        raise ConfigError("config.json must name its model in architectures[0] or architecture",
                           known=registered_architectures())
     arch = _ARCHITECTURES.get(names[0])
     if arch is None:

@@ -40,6 +40,30 @@ class RopeSpec:
 
 
 @dataclass(frozen=True)
+class ScaledRopeSpec:
+    """Rotary encoding whose slow pairs are slowed for contexts longer than the frequencies were chosen for.
+
+    Pair ``i`` of ``rotary_dim / 2`` turns by ``f_i = theta^(-2i/rotary_dim)`` a position.  With
+    ``pair_of(t) = rotary_dim ln(original / (2 pi t)) / (2 ln theta)`` (the pair that makes ``t`` turns over
+    ``original`` positions), ``lo = max(floor(pair_of(fast)), 0)``, ``hi = min(ceil(pair_of(slow)), rotary_dim - 1)``
+    and ``ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)`` the frequency becomes
+    ``f_i / factor * ramp_i + f_i (1 - ramp_i)``, and cos and sin are both multiplied by
+    ``amplitude_slope * ln(factor) + 1``.  ``factor = None``: plain rotation."""
+
+    head_dim: int
+    rotary_dim: int
+    theta: float
+    max_position: int
+    factor: Optional[float] = None
+    original: float = 0.0
+    fast: float = 32.0
+    slow: float = 1.0
+    amplitude_slope: float = 0.1
+    layout: str = "half"
+    kind: str = "scaled_rope"
+
+
+@dataclass(frozen=True)
 class NoPositionSpec:
     kind: str = "none"
 
@@ -59,6 +83,29 @@ class AttentionSpec:
 
 
 @dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention through low-rank bottlenecks: queries from a normed latent of ``q_rank`` features; keys and values
+    of all heads from one normed latent row of ``kv_rank`` features per token, plus ``rot_dim`` rotated key features
+    that all heads share.  A head has ``plain_dim`` unrotated and ``rot_dim`` rotated query/key features (in that
+    order) and ``value_dim`` value features.  ``gated``: head ``h``'s output is multiplied by
+    ``sigmoid(W_g x)[h]``.  ``position`` is the encoding of the ``rot_dim`` part (its ``head_dim`` = ``rot_dim``)."""
+
+    hidden: int
+    n_heads: int
+    plain_dim: int
+    rot_dim: int
+    value_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    eps: float                         # of the two latent norms
+    position: Any
+    window: Optional[int] = None       # keys a query sees, itself included; None = all
+    gated: bool = True
+    kind: str = "latent_attention"
+
+
+@dataclass(frozen=True)
 class ShortConvSpec:
     hidden: int
     width: int                         # taps, the current input included (conv_L_cache)
@@ -71,6 +118,23 @@ class SwiGLUSpec:
     hidden: int
     intermediate: int
     kind: str = "swiglu"
+
+
+@dataclass(frozen=True)
+class TableMoESpec:
+    """A mixture of small feed-forwards whose routing is a table: token id ``v`` uses the ``top`` experts
+    ``table[v, :]``, each with weight ``1 / top``.  An expert is ``W_down act(W_up x)``, ``act`` the square of relu.
+    ``shared_ff``: a further expert of that width runs for every token, scaled by ``sigmoid(w_gate . x)`` when
+    ``shared_gate`` (None: no shared expert)."""
+
+    hidden: int
+    vocab: int
+    n_experts: int
+    top: int
+    expert_ff: int
+    shared_ff: Optional[int] = None
+    shared_gate: bool = True
+    kind: str = "table_moe"
 
 
 @dataclass(frozen=True)
@@ -88,6 +152,20 @@ class BlockSpec:
     ffn_norm: Any
     names: Mapping[str, str] = field(compare=False, hash=False, default_factory=dict)
     kind: str = "prenorm"
+
+
+@dataclass(frozen=True)
+class OutNormBlockSpec:
+    """One block whose norms stand on the sub-layers' outputs: ``h += mult * norm_a(mixer(h));
+    h += mult * norm_b(ffn(h))``; the sub-layers read ``h`` itself.  ``names`` as in :class:`BlockSpec`."""
+
+    mixer: Any
+    mixer_norm: Any
+    ffn: Any                           # None = no feed-forward in this block
+    ffn_norm: Any
+    mult: float = 1.0
+    names: Mapping[str, str] = field(compare=False, hash=False, default_factory=dict)
+    kind: str = "outnorm"
 
 
 @dataclass(frozen=True)

@@ -19,7 +19,7 @@ void gs_set_error(const char* fmt, ...) {
 
 extern "C" const char* gs_last_error() { return g_err; }
 
-extern "C" int gs_abi_version() { return 9; }
+extern "C" int gs_abi_version() { return 10; }
 
 // ------------------------------------------------------------------ embedding
 
@@ -380,6 +380,57 @@ extern "C" int gs_residual_add(float* res, const void* delta, int delta_dtype, l
   else
     GS_REQUIRE(false, "residual_add: unknown dtype %d", delta_dtype);
   GS_LAUNCH_CHECK("residual_add");
+  return 0;
+}
+
+// A block whose norm stands on its sub-layer's output: res[t, :] += mult * y[t, :] * inv_rms(y[t, :]) * w, and the new
+// row also in the activation type (`rows`, what the next sub-layer's products read).  y == nullptr: nothing is
+// added, the rows are only copied out (the first sub-layer's input).  All arithmetic float32; one block per row.
+template <typename TY, typename TO>
+__global__ void norm_scaled_add_kernel(float* __restrict__ res, const TY* __restrict__ y, const float* __restrict__ w,
+                                       float eps, float mult, TO* __restrict__ rows, int H) {
+  __shared__ float red[17];
+  const int t = blockIdx.x;
+  float* r = res + (size_t)t * H;
+  if (y) {
+    const TY* yr = y + (size_t)t * H;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) {
+      const float v = to_f32(yr[j]);
+      ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float inv = norm_inverse(ss, (float)H, eps);
+    for (int j = threadIdx.x; j < H; j += blockDim.x) {
+      const float v = r[j] + mult * (to_f32(yr[j]) * inv * w[j]);
+      r[j] = v;
+      if (rows) rows[(size_t)t * H + j] = from_f32<TO>(v);
+    }
+  } else if (rows) {
+    for (int j = threadIdx.x; j < H; j += blockDim.x) rows[(size_t)t * H + j] = from_f32<TO>(r[j]);
+  }
+}
+
+extern "C" int gs_norm_scaled_add(float* res, const void* y, int y_dtype, const float* w, float eps, float mult,
+                                  void* rows, int rows_dtype, int T, int H, hipStream_t stream) {
+  GS_REQUIRE(T >= 0 && H > 0, "norm_scaled_add: bad sizes T=%d H=%d", T, H);
+  GS_REQUIRE(y == nullptr || (w != nullptr && eps > 0.f), "norm_scaled_add: a norm needs its weight and a positive eps");
+  if (T == 0) return 0;
+  const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
+#define GS_RUN(TY, TO) \
+  norm_scaled_add_kernel<TY, TO><<<T, threads, 0, stream>>>(res, (const TY*)y, w, eps, mult, (TO*)rows, H)
+  if (y_dtype == GS_F32 && rows_dtype == GS_F32)
+    GS_RUN(float, float);
+  else if (y_dtype == GS_BF16 && rows_dtype == GS_BF16)
+    GS_RUN(bf16, bf16);
+  else if (y_dtype == GS_F32 && rows_dtype == GS_BF16)
+    GS_RUN(float, bf16);
+  else if (y_dtype == GS_BF16 && rows_dtype == GS_F32)
+    GS_RUN(bf16, float);
+  else
+    GS_REQUIRE(false, "norm_scaled_add: unknown dtypes %d %d", y_dtype, rows_dtype);
+#undef GS_RUN
+  GS_LAUNCH_CHECK("norm_scaled_add");
   return 0;
 }
 

@@ -883,3 +883,141 @@ def attention_prefill_wide(q, q_stride, kcache, vcache, positions, tiles, block_
                                            block_table.shape[1], page_size, kcache.shape[0],
                                            window or 0, scale, _p(out), nh, nkv, d, rows, key_splits, _stream()))
     return out
+
+
+# ---------------------------------------------------------------------- blocks with their norm on the output
+
+def norm_scaled_add(res: torch.Tensor, y, weight, eps: float, mult: float, rows_dtype=None) -> torch.Tensor:
+    """``res += mult * rmsnorm(y) * weight`` row by row (``y = None``: nothing is added); returns the stream's new rows
+    in ``rows_dtype`` (what the next sub-layer's products read), or None when no type is given."""
+    _dev(res, y, weight)
+    _need(res.dtype == torch.float32 and res.dim() == 2, "norm_scaled_add: the residual stream is float32 (T, H)")
+    T, H = res.shape
+    _need(y is None or (y.shape == res.shape and weight is not None and weight.dtype == torch.float32
+                        and weight.shape == (H,)), "norm_scaled_add: y has the stream's shape, weight is float32 (H,)")
+    rows = None if rows_dtype is None else torch.empty((T, H), dtype=rows_dtype, device=res.device)
+    _check(lib().gs_norm_scaled_add(_p(res), _p(y), _dt(y) if y is not None else _dt(rows), _p(weight), float(eps),
+                                    float(mult), _p(rows), _dt(rows) if rows is not None else _dt(y), T, H, _stream()))
+    return rows
+
+
+# ---------------------------------------------------------------------- attention through a cached latent row
+
+def latent_prep(down, q_off, q_rank, kv_off, c, r, q_weight, kv_weight, eps, cos, sin, positions, seq_of_token,
+                block_table, page_size, cache, write_kv: bool = True) -> torch.Tensor:
+    """Per token of ``down (T, ld)``: the columns ``[q_off, q_off + q_rank)`` RMS-normed with ``q_weight`` are
+    returned as ``(T, q_rank)``; the columns ``[kv_off, kv_off + c)`` RMS-normed with ``kv_weight`` and the ``r``
+    columns behind them, rotated by the token's position, are written into the token's cache row ``[c | r]``.
+    ``cache (pages, 1, page_size, c + r)``."""
+    _dev(down, q_weight, kv_weight, positions, seq_of_token, block_table, cache)
+    T, ld = down.shape
+    _need(cache.dtype == down.dtype and cache.dim() == 4 and cache.shape[1:] == (1, page_size, c + r),
+          "latent_prep: the cache is (pages, 1, page_size, c + r) in the activations' type")
+    _need(q_weight.dtype == torch.float32 and q_weight.shape == (q_rank,) and kv_weight.dtype == torch.float32
+          and kv_weight.shape == (c,), "latent_prep: norm weights are float32 (q_rank,), (c,)")
+    if r:
+        _dev(cos, sin)
+        _need(cos.dtype == torch.float32 and sin.shape == cos.shape and cos.dim() == 2 and cos.shape[1] == r // 2,
+              "latent_prep: cos and sin are float32 (positions, r / 2)")
+    _i32(positions, T, "positions")
+    _i32(seq_of_token, T, "seq_of_token")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (nseq, max_blocks)")
+    a = torch.empty((T, q_rank), dtype=down.dtype, device=down.device)
+    _check(lib().gs_latent_prep(_p(down), _dt(down), ld, q_off, q_rank, kv_off, c, r, _p(q_weight), _p(kv_weight),
+                                float(eps), _p(cos) if r else None, _p(sin) if r else None, _p(positions),
+                                _p(seq_of_token), _p(block_table), block_table.shape[1], page_size, _p(cache), _p(a),
+                                1 if write_kv else 0, T, _stream()))
+    return a
+
+
+def latent_q_rot(q, H, n, r, c, cos, sin, positions, qa) -> None:
+    """The last ``r`` features of every head of ``q (T, H (n + r))``, rotated by the token's position, into
+    ``qa (T, H (c + r))`` behind each head's first ``c`` columns."""
+    _dev(q, positions, qa)
+    T = q.shape[0]
+    _need(q.shape == (T, H * (n + r)) and qa.shape == (T, H * (c + r)) and qa.dtype == q.dtype,
+          "latent_q_rot: q is (T, H (n + r)), qa (T, H (c + r)) of one type")
+    _i32(positions, T, "positions")
+    if r == 0:
+        return
+    _dev(cos, sin)
+    _need(cos.dtype == torch.float32 and sin.shape == cos.shape and cos.dim() == 2 and cos.shape[1] == r // 2,
+          "latent_q_rot: cos and sin are float32 (positions, r / 2)")
+    _check(lib().gs_latent_q_rot(_p(q), _dt(q), q.stride(0), H, n, r, c, _p(cos), _p(sin), _p(positions), _p(qa), T,
+                                 _stream()))
+
+
+def heads_product(x, hx: int, w, y, hy: int, K: int, gate=None) -> torch.Tensor:
+    """``y[t, h hy : h hy + N] = w[h] @ x[t, h hx : h hx + K]`` for every head ``h`` of ``w (H, N, K)``, float32 sums in
+    a fixed order; with ``gate (T, >= H)`` the result of head ``h`` is multiplied by ``sigmoid(gate[t, h])``."""
+    _need(x.is_cuda and y.is_cuda and w.is_cuda and w.is_contiguous() and x.dim() == 2 and y.dim() == 2
+          and x.stride(1) == 1 and y.stride(1) == 1, "heads_product: rows with unit column stride, on the GPU")
+    H, N, Kw = w.shape
+    _need(Kw == K and x.shape[0] == y.shape[0] and y.dtype == x.dtype, "heads_product: shapes or types differ")
+    M = x.shape[0]
+    ldg = 0
+    if gate is not None:
+        _need(gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[0] == M and gate.shape[1] >= H
+              and gate.dtype == x.dtype, "heads_product: the gate is (T, >= H) of the rows' type")
+        ldg = gate.stride(0) if M > 1 else gate.shape[1]
+    _check(lib().gs_heads_product(_p(x), _dt(x), x.stride(0) if M > 1 else x.shape[1], hx, _p(w), _dt(w), _p(y),
+                                  y.stride(0) if M > 1 else y.shape[1], hy, _p(gate), ldg, M, N, K, H, _stream()))
+    return y
+
+
+def attention_latent(qa, cache, positions, seq_of_token, block_table, page_size, window, scale, H, c, r, ntok,
+                     out: torch.Tensor = None) -> torch.Tensor:
+    """Attention of ``qa (T, H (c + r))`` over cached rows ``[c | r]``: scores over all ``c + r`` columns, the output
+    ``(T, H c)`` a softmax-weighted sum of the rows' first ``c`` columns.  Any sizes, float32 arithmetic."""
+    _dev(qa, cache, positions, seq_of_token, block_table, out)
+    _need(qa.shape == (ntok, H * (c + r)) and cache.dtype == qa.dtype, "attention_latent: qa is (T, H (c + r)) in the cache's type")
+    _need(cache.dim() == 4 and cache.shape[1:] == (1, page_size, c + r), "attention_latent: the cache is (pages, 1, page_size, c + r)")
+    _i32(positions, ntok, "positions")
+    _i32(seq_of_token, ntok, "seq_of_token")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (nseq, max_blocks)")
+    if out is None:
+        out = torch.empty((ntok, H * c), dtype=qa.dtype, device=qa.device)
+    _need(out.shape == (ntok, H * c) and out.dtype == qa.dtype, "attention_latent: out has the wrong shape or type")
+    _check(lib().gs_attention_latent(_p(qa), _p(cache), _dt(qa), _p(positions), _p(seq_of_token), _p(block_table),
+                                     block_table.shape[1], page_size, window or 0, float(scale), _p(out), ntok, H, c, r,
+                                     _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------- feed-forwards routed by a table
+
+def relu_squared(x: torch.Tensor, F: int) -> torch.Tensor:
+    """``relu(x[:, :F])^2`` as contiguous rows ``(T, F)``."""
+    _need(x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and x.shape[1] >= F, "relu_squared: rows (T, >= F) on the GPU")
+    T = x.shape[0]
+    out = torch.empty((T, F), dtype=x.dtype, device=x.device)
+    _check(lib().gs_relu_squared(_p(x), _dt(x), x.stride(0) if T > 1 else x.shape[1], _p(out), T, F, _stream()))
+    return out
+
+
+def moe_table(x, ids, table, up, down, shared=None, gate=None) -> torch.Tensor:
+    """``y[t] = (1 / top) sum_k down[e_k] relu(up[e_k] x[t])^2`` with ``e_k = table[ids[t], k]``; ``up (E, F, H)``,
+    ``down (E, H, F)``, ``table (vocab, top)`` int32.  With ``shared (T, H)`` and ``gate`` (one number a token, the
+    first column of its rows): ``+ sigmoid(gate[t]) * shared[t]``.  Token by token: only the chosen experts' weights
+    are read."""
+    _dev(ids, table, up, down, shared)
+    _need(x.is_cuda and x.dim() == 2 and x.stride(1) == 1, "moe_table: rows (T, H) on the GPU")
+    T, H = x.shape
+    E, F, Hw = up.shape
+    _need(Hw == H and down.shape == (E, H, F) and up.dtype == down.dtype, "moe_table: up is (E, F, H), down (E, H, F)")
+    _need(table.dtype == torch.int32 and table.dim() == 2, "moe_table: the table is int32 (vocab, top)")
+    top = table.shape[1]
+    _i32(ids, T, "token ids")
+    ldg = 0
+    if shared is not None:
+        _need(shared.shape == (T, H) and shared.dtype == x.dtype and gate is not None and gate.is_cuda and gate.dim() == 2
+              and gate.shape[0] == T and gate.dtype == x.dtype and gate.stride(1) == 1,
+              "moe_table: shared rows (T, H) come with a gate (T, >= 1) of the rows' type")
+        ldg = gate.stride(0) if T > 1 else gate.shape[1]
+    a = torch.empty((T, top, F), dtype=x.dtype, device=x.device)
+    y = torch.empty((T, H), dtype=x.dtype, device=x.device)
+    _check(lib().gs_moe_table_up(_p(x), _dt(x), x.stride(0) if T > 1 else H, _p(ids), _p(table), top, _p(up), _dt(up), F,
+                                 H, _p(a), T, _stream()))
+    _check(lib().gs_moe_table_down(_p(a), _dt(a), _p(ids), _p(table), top, _p(down), _dt(down), F, H, _p(shared),
+                                   _p(gate) if shared is not None else None, ldg, _p(y), T, _stream()))
+    return y

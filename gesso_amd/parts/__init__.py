@@ -1,5 +1,5 @@
-from . import attention, block, rmsnorm, rope, shortconv, swiglu  # noqa: F401  (registers the kinds)
-from .base import MATRIX, TABLE, VECTOR, PagedKV, Part, SlotState, TensorSpec
+from . import attention, block, latent_attention, rmsnorm, rope, shortconv, swiglu, table_moe  # noqa: F401  (registers the kinds)
+from .base import INDEX, MATRIX, TABLE, VECTOR, PagedKV, Part, SlotState, TensorSpec
 from .registry import build, part_class, register, unregister
 from .rmsnorm import ResidualStream
 from .runtime import DeferredLinear, Runtime, RuntimeOptions

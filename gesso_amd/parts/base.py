@@ -31,13 +31,16 @@ from typing import Dict, Optional, Tuple
 MATRIX = "matrix"     # operand of a matrix product: keeps the stored width (bfloat16 stays bfloat16)
 VECTOR = "vector"     # norm weights, taps, biases: held in float32 (an exact widening)
 TABLE = "table"       # embedding table; a matrix that is also gathered from
+INDEX = "index"       # a table of integers (which experts a token id uses): held as int32
 
 
 @dataclass(frozen=True)
 class TensorSpec:
     shape: Tuple[int, ...]
     role: str = MATRIX
-    init: str = "normal"          # "normal": N(0, std); "one_plus_normal": 1 + N(0, std)
+    init: str = "normal"          # "normal": N(0, std); "one_plus_normal": 1 + N(0, std);
+                                  # "distinct": integers below ``high``, those of a row all different
+    high: int = 0
 
 
 @dataclass(frozen=True)

@@ -85,4 +85,37 @@ class PreNormBlock(Part):
         return all(getattr(p, "graph_safe", False) for p in parts)
 
 
+class OutNormBlock(PreNormBlock):
+    """``h += mult * norm_a(mixer(h)); h += mult * norm_b(ffn(h))``: the norms stand on the sub-layers' outputs, the
+    sub-layers read the stream itself (in the activation type).  The add, the norm and the rows for the next
+    sub-layer are one kernel."""
+
+    first_norm = None           # nothing norms the stream before this block's mixer reads it
+
+    def forward(self, stream, ctx, cache):
+        rt, ops, s = self.rt, self.rt.ops, self.spec
+        rows_dtype = None if rt.dtype == stream.res.dtype else rt.dtype
+        stream.flush(rt)
+        x = stream.rows
+        if x is None:
+            x = stream.res if rows_dtype is None else ops.norm_scaled_add(stream.res, None, None, 0.0, 0.0, rows_dtype)
+        with rt.stage(getattr(self.mixer, "stage", "mixer")):
+            y = rt.dense(self.mixer.forward(x, ctx, cache))
+        with rt.stage("norm"):
+            x = ops.norm_scaled_add(stream.res, y, self.mixer_norm.weight, self.mixer_norm.spec.eps, s.mult, rows_dtype)
+        if self.ffn is not None:
+            with rt.stage(getattr(self.ffn, "stage", "ffn")):
+                y = rt.dense(self.ffn.forward(stream.res if rows_dtype is None else x, ctx))
+            with rt.stage("norm"):
+                x = ops.norm_scaled_add(stream.res, y, self.ffn_norm.weight, self.ffn_norm.spec.eps, s.mult, rows_dtype)
+        # what earlier writers left beside the stream (sums of squares, pre-weighted rows) no longer describes it
+        stream.pending = stream.ssq = stream.xs = stream.xs_for = stream.normed = None
+        stream.rows = x
+
+    @property
+    def portions_recordable(self) -> bool:
+        return False
+
+
 register("block", "prenorm", PreNormBlock)
+register("block", "outnorm", OutNormBlock)

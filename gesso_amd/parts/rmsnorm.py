@@ -24,7 +24,7 @@ class ResidualStream:
     in bfloat16, and the norm's consumer needs no norm pass at all.  ``xs_for`` is the norm ``xs`` was made for.
     """
 
-    __slots__ = ("res", "pending", "ssq", "xs", "xs_for", "following", "normed")
+    __slots__ = ("res", "pending", "ssq", "xs", "xs_for", "following", "normed", "rows")
 
     def __init__(self, res, pending=None, ssq=None, xs=None, xs_for=None):
         self.res = res
@@ -33,11 +33,12 @@ class ResidualStream:
         self.xs, self.xs_for = xs, xs_for
         self.following = None
         self.normed = None            # the rows normed for ``xs_for``, where the last push made them
+        self.rows = None              # the stream itself in the activation type, where the last writer left it
 
     def push(self, out, rt, next_norm=None) -> None:
         from .runtime import DeferredLinear
         self.flush(rt)
-        self.xs = self.xs_for = self.normed = None
+        self.xs = self.xs_for = self.normed = self.rows = None
         if isinstance(out, DeferredLinear) and self.res.shape[0] > rt.weighted_rows_max:
             # many rows: K is shared out over many blocks, and the pass that adds their partial sums to the stream
             # norms the rows for the next norm on its way (it sees whole rows)
@@ -64,7 +65,7 @@ class ResidualStream:
         if self.pending is not None:
             rt.ops.residual_add(self.res, self.pending)
             self.pending, self.ssq = None, None
-            self.xs = self.xs_for = self.normed = None
+            self.xs = self.xs_for = self.normed = self.rows = None
 
 
 def row_weight_of(norm, res, rt):

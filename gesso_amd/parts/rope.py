@@ -42,6 +42,51 @@ class Rope(Part):
         self.cos, self.sin = rt.shared(("rope", spec.rotary_dim, float(spec.theta), spec.max_position), make)
 
 
+def scaled_rope_tables(spec):
+    """cos and sin tables of a :class:`~gesso_amd.config.spec.ScaledRopeSpec` (see there for the rule): pairs that turn
+    often keep their frequency, slow pairs are slowed by ``factor``, those between are blended, and both tables carry
+    the amplitude factor.  float64 on the host, stored as float32."""
+    import math
+    dims, theta = spec.rotary_dim, float(spec.theta)
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    freq = torch.tensor(theta, dtype=torch.float64) ** (-2.0 * i / dims)
+    amplitude = 1.0
+    if spec.factor is not None:
+        def pair_of(turns):
+            return dims * math.log(float(spec.original) / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+        lo = max(math.floor(pair_of(float(spec.fast))), 0)
+        hi = min(math.ceil(pair_of(float(spec.slow))), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        freq = freq / float(spec.factor) * ramp + freq * (1.0 - ramp)
+        amplitude = float(spec.amplitude_slope) * math.log(float(spec.factor)) + 1.0
+    ang = torch.arange(spec.max_position, dtype=torch.float64)[:, None] * freq[None, :]
+    return (torch.cos(ang) * amplitude).to(torch.float32), (torch.sin(ang) * amplitude).to(torch.float32)
+
+
+class ScaledRope(Part):
+    """Rotation with slowed pairs and an amplitude: the same three attributes as :class:`Rope`, other tables."""
+
+    graph_safe = True
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        if spec.rotary_dim % 2 or not 0 <= spec.rotary_dim <= spec.head_dim:
+            raise ValueError(f"rotary_dim {spec.rotary_dim} must be even and within the head width {spec.head_dim}")
+        self.rotary_dim = spec.rotary_dim
+        self.layout = spec.layout
+        if self.layout not in rt.ops.ROPE_LAYOUTS:
+            raise ValueError(f"rotation pairs are laid out 'half' or 'interleaved', not {self.layout!r}")
+        self.cos = self.sin = None
+        if spec.rotary_dim:
+            def make():
+                cos, sin = scaled_rope_tables(spec)
+                return cos.to(rt.device), sin.to(rt.device)
+
+            key = ("scaled_rope", spec.rotary_dim, float(spec.theta), spec.max_position, spec.factor, float(spec.original),
+                   float(spec.fast), float(spec.slow), float(spec.amplitude_slope))
+            self.cos, self.sin = rt.shared(key, make)
+
+
 class NoPosition(Part):
     graph_safe = True
     rotary_dim = 0
@@ -51,4 +96,5 @@ class NoPosition(Part):
 
 
 register("position", "rope", Rope)
+register("position", "scaled_rope", ScaledRope)
 register("position", "none", NoPosition)

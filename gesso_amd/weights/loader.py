@@ -8,8 +8,8 @@ one (``src/Inference/materialize_architecture.jl:217-222``, ``:344-349``, ``:369
 Storage widths: in ``bfloat16`` mode a matrix stored in bfloat16 stays bfloat16 and a matrix
 stored in 32-bit stays 32-bit (its products then run in float32); half precision and float64
 become float32.  Small vectors (norm weights, taps, biases) are held in float32, an exact
-widening of bfloat16.  In ``float32`` mode everything is widened to float32.  Integer tables
-would be kept as int32.  A tied head may be present in the file if it equals the embedding
+widening of bfloat16.  In ``float32`` mode everything is widened to float32.  Integer tables (a part
+declares them with the role ``INDEX``) are kept as int32.  A tied head may be present in the file if it equals the embedding
 table (``materialize_architecture.jl:268-289``).
 """
 from __future__ import annotations
@@ -20,7 +20,7 @@ from typing import Dict, Iterable
 import torch
 
 from ..errors import WeightError
-from ..parts.base import VECTOR, TensorSpec
+from ..parts.base import INDEX, VECTOR, TensorSpec
 from .safetensors_io import open_model_files, write_safetensors
 
 _FLOATS = (torch.float64, torch.float32, torch.float16, torch.bfloat16)
@@ -56,7 +56,7 @@ def load_tensors(model_dir: str, table: Dict[str, TensorSpec], mode: torch.dtype
             f = where[name]
             if _core(f.shape(name)) != _core(ts.shape):
                 wrong_shape.append(f"{name}: file has {tuple(f.shape(name))}, the configuration needs {tuple(ts.shape)}")
-            if f.dtype(name) not in _FLOATS:
+            if f.dtype(name) not in (_INTS if ts.role == INDEX else _FLOATS):
                 wrong_type.append(f"{name}: {f.dtype(name)}")
     if missing or unexpected or wrong_shape or wrong_type or duplicates:
         parts = []
@@ -106,6 +106,12 @@ def random_tensors(table: Dict[str, TensorSpec], seed: int, dtype: torch.dtype, 
     out = {}
     for name, ts in table.items():
         t = torch.empty(ts.shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
+        if ts.init == "distinct":
+            # a row's entries: the first of a random order of 0 .. high - 1
+            rows, n = int(torch.tensor(ts.shape[:-1]).prod()) if len(ts.shape) > 1 else 1, ts.shape[-1]
+            order = torch.rand((rows, ts.high), generator=gen, device=device).argsort(dim=1)
+            out[name] = order[:, :n].reshape(ts.shape).to(torch.int32)
+            continue
         if ts.init == "one_plus_normal":
             t += 1.0
         elif ts.init != "normal":
