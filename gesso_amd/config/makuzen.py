@@ -14,7 +14,7 @@ would be a mechanism it does not compute); a key whose value is null counts as l
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Optional, Tuple
 
 from ..errors import ConfigError
@@ -166,7 +166,8 @@ class MakuzenConfig:
     embedding_scale: float = 1.0
     norm_eps: float = 1e-5
     residual_mult: float = 1.0
-    max_position: int = DEFAULT_MAX_POSITION     # not a key of the file: what the rotation tables are made for
+    # not a key of the file (and no part of what makes two configurations equal): what the rotation tables are made for
+    max_position: int = field(default=DEFAULT_MAX_POSITION, compare=False)
 
     def __post_init__(self):
         if self.vocab < 1 or self.width < 1:

@@ -4,7 +4,7 @@ Nothing is imported from ``gesso_amd``: a model folder is read with ``json`` and
 package, the arithmetic is explicit torch on the CPU in float64 (or another type on request).  One
 function per mechanism:
 
-    embedding  rmsnorm  yarn_frequencies  rotate  latent_attention  expert  table_moe  layer  forward
+    embedding  rmsnorm  yarn_frequencies  rotate  windowed_attention  latent_attention  expert  table_moe  layer  forward
 
 Notation.  Rows are tokens: activations are ``(T, features)``, a linear weight ``W`` is ``(out, in)``
 and acts as ``y = x @ W.T``.  ``rms(x) = x / sqrt(mean(x^2) + eps)`` with eps under the root.
@@ -108,9 +108,24 @@ def rotate(x: torch.Tensor, positions, freqs, mult: float) -> torch.Tensor:
     return out
 
 
+def windowed_attention(q_plain, q_rot, k_plain, k_rot, v, scale: float, window=None) -> torch.Tensor:
+    """Softmax attention of token ``i`` over the tokens ``j`` with ``0 <= i - j < window`` (all ``j <= i`` without a
+    window).  ``q_plain, k_plain (T, H, n)``, ``q_rot (T, H, r)``, ``k_rot (T, r)`` shared by the heads,
+    ``v (T, H, dv)``; the score is ``(q_plain . k_plain + q_rot . k_rot) * scale``.  Returns ``(T, H, dv)``."""
+    T, H = q_plain.shape[0], q_plain.shape[1]
+    out = torch.zeros(T, H, v.shape[2], dtype=v.dtype)
+    for i in range(T):
+        lo = 0 if not window else max(0, i - int(window) + 1)
+        for h in range(H):
+            s = (k_plain[lo:i + 1, h] @ q_plain[i, h] + k_rot[lo:i + 1] @ q_rot[i, h]) * scale
+            pr = torch.softmax(s, dim=0)
+            out[i, h] = pr @ v[lo:i + 1, h]
+    return out
+
+
 def latent_attention(x, w, p, mx, eps, positions, store=_keep):
-    """The mixer on ``x (T, width)``; ``w``: name -> tensor, ``p``: the tensors' prefix (``l3.mix``), ``mx``: the
-    layer's ``mixer`` entry of the configuration."""
+    """The mixer on ``x (T, width)``, the whole sequence from position 0; ``w``: name -> tensor, ``p``: the tensors'
+    prefix (``l3.mix``), ``mx``: the layer's ``mixer`` entry of the configuration."""
     T = x.shape[0]
     H, n, r, dv, c = int(mx["heads"]), int(mx["dim"]), int(mx["rot_dim"]), int(mx["vdim"]), int(mx["kv_rank"])
     rot = mx.get("rot") or {}
@@ -129,14 +144,7 @@ def latent_attention(x, w, p, mx, eps, positions, store=_keep):
     k_plain = store(linear(z, w[p + ".uk"])).reshape(T, H, n)
     v = store(linear(z, w[p + ".uv"])).reshape(T, H, dv)
     gate = torch.sigmoid(linear(x, w[p + ".g"]))                       # (T, H)
-
-    out = torch.zeros(T, H, dv, dtype=x.dtype)
-    for i in range(T):
-        lo = 0 if not window else max(0, i - int(window) + 1)
-        for h in range(H):
-            s = (k_plain[lo:i + 1, h] @ q_plain[i, h] + k_rot[lo:i + 1] @ q_rot[i, h]) * scale
-            pr = torch.softmax(s, dim=0)
-            out[i, h] = pr @ v[lo:i + 1, h]
+    out = windowed_attention(q_plain, q_rot, k_plain, k_rot, v, scale, window)
     out = store(out * gate[:, :, None])
     return store(linear(out.reshape(T, H * dv), w[p + ".o"]))
 
