@@ -1,0 +1,229 @@
+// Attention over cached latent rows on the matrix cores (bfloat16 storage): prompt portions and single tokens alike.
+//
+// Every head of a token attends over the same rows [z | k_rot] (D = c + r columns; the first c are also the values),
+// so what a block shares through LDS is one tile of rows for all of its queries: a block owns up to 64 query rows
+// (token, head) of one sequence, consecutive tokens x up to 64 heads, 16 rows a wavefront; a step stages KSTEP cached
+// rows once, row-major for the score product and transposed (column-major) for the value product.
+//
+// Both products are computed transposed (v_mfma_f32_16x16x32_bf16), so that all a lane holds concerns one query row
+// (lane % 16) and no softmax weight crosses lanes:
+//   S^T = R Q^T     A = staged rows (lane l: row l % 16 of a block of 16, columns 8 (l / 16) .. + 7 of a step of 32),
+//                   B = the wavefront's query fragments (registers); lane l gets rows 4 (l / 16) + 0..3 of the block.
+//   O^T = Z^T P^T   B = the lane's own eight weights of a chunk of 32 rows (two blocks of four), A = the transposed
+//                   values read in the same order; lane l gets value columns 4 (l / 16) + 0..3 of a tile of 16.
+// Scores, maxima, sums and softmax weights are float32.  A weight enters the matrix cores as the sum of two bfloat16
+// numbers (its rounding and the rounding of what that left over), two products a chunk: the weights keep 16 bits
+// of mantissa, and the sums are float32.
+//
+// The query at position p sees rows lo..p of its sequence, lo = 0 or p - window + 1; a block walks from the oldest row
+// any of its queries sees to its last query's own, each row masked per query.  Rows past the block's last are staged
+// as zeros (their pages may belong to nobody).
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
+
+#define LM_LOG2E 1.4426950408889634f
+#define LM_ROWS 64     // query rows a block
+
+// CT: the most tiles of 16 value columns (c <= 16 CT); the score product takes up to CT / 2 + 2 steps of 32 columns.
+template <int CT, int KSTEP>
+__global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
+    const bf16* __restrict__ qa, const bf16* __restrict__ cache, const int* __restrict__ positions,
+    const int* __restrict__ tile_seq, const int* __restrict__ tile_row, const int* __restrict__ tile_n,
+    const int* __restrict__ block_table, int max_blocks, int page_size, int window, float scale,
+    bf16* __restrict__ out, int H, int HB, int c, int D) {
+  constexpr int DK = CT / 2 + 2;
+  constexpr int NB = KSTEP / 16, NC = KSTEP / 32, VROW = KSTEP + 4;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int Dp = (D + 31) & ~31, krow = Dp + 8;
+  bf16* ks = reinterpret_cast<bf16*>(lds);                                            // [KSTEP][krow]
+  uint16_t* vt = reinterpret_cast<uint16_t*>(lds + (size_t)KSTEP * krow * 2);         // [c][VROW]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r16 = lane & 15, g = lane >> 4;
+  const int tile = blockIdx.x;
+  int seq = tile, row0 = tile, nt = 1;               // without a list: sequence i brings the single token i
+  if (tile_seq) {
+    seq = tile_seq[tile];
+    row0 = tile_row[tile];
+    nt = tile_n[tile];
+  }
+  const int h0 = blockIdx.y * HB;
+  const int hb = H - h0 < HB ? H - h0 : HB;
+  const int nrows = nt * hb;
+  const int pos0 = positions[row0];                  // a tile's tokens stand at consecutive positions
+  const int* bt = block_table + (size_t)seq * max_blocks;
+  const int m = wave * 16 + r16;
+  const bool valid = m < nrows;
+  const int ti = valid ? m / hb : 0, head = h0 + (valid ? m % hb : 0);
+  const int pos = pos0 + ti;
+  const size_t qrow = (size_t)(row0 + ti) * H + head;
+  const bool wave_on = wave * 16 < nrows;
+  const int ti_lo = (wave * 16) / hb;
+  const int ti_hi = (wave * 16 + 15) / hb < nt - 1 ? (wave * 16 + 15) / hb : nt - 1;
+
+  bf16x8_t qf[DK];
+#pragma unroll
+  for (int kk = 0; kk < DK; ++kk) {
+    const int f = 32 * kk + 8 * g;
+    u32x4_t v = {0u, 0u, 0u, 0u};
+    if (valid && f < D) v = *reinterpret_cast<const u32x4_t*>(qa + qrow * D + f);
+    qf[kk] = __builtin_bit_cast(bf16x8_t, v);
+  }
+  f32x4_t acc[CT];
+#pragma unroll
+  for (int dt = 0; dt < CT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float mrun = -INFINITY, lrun = 0.f;
+  const float sc = scale * LM_LOG2E;
+  const int kmax = pos0 + nt - 1;
+  const int kmin = window > 0 ? (pos0 - window + 1 > 0 ? pos0 - window + 1 : 0) : 0;
+  const int chunks = Dp >> 3, ct = c >> 4;
+
+  for (int s0 = kmin; s0 <= kmax; s0 += KSTEP) {
+    __syncthreads();
+    for (int idx = tid; idx < KSTEP * chunks; idx += 256) {
+      const int kk = idx / chunks, f = (idx - kk * chunks) * 8;
+      const int j = s0 + kk;
+      u32x4_t v = {0u, 0u, 0u, 0u};
+      if (j <= kmax && f < D) {
+        const int page = bt[j / page_size];
+        v = *reinterpret_cast<const u32x4_t*>(cache + ((size_t)page * page_size + j % page_size) * D + f);
+      }
+      *reinterpret_cast<u32x4_t*>(ks + (size_t)kk * krow + f) = v;
+      if (f < c) {
+        const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          vt[(size_t)(f + 2 * e) * VROW + kk] = (uint16_t)(w[e] & 0xffffu);
+          vt[(size_t)(f + 2 * e + 1) * VROW + kk] = (uint16_t)(w[e] >> 16);
+        }
+      }
+    }
+    __syncthreads();
+    // a wavefront none of whose queries sees a row of this step waits for the next
+    const bool step_on = wave_on && s0 <= pos0 + ti_hi && (window <= 0 || s0 + KSTEP - 1 > pos0 + ti_lo - window);
+    if (!step_on) continue;
+    f32x4_t st[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      st[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < DK; ++kk)
+        if (32 * kk < D) {
+          const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks + (size_t)(16 * b + r16) * krow + 32 * kk + 8 * g);
+          st[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[kk], st[b], 0, 0, 0);
+        }
+    }
+    float mstep = -INFINITY;
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int j = s0 + 16 * b + 4 * g + e;
+        const bool seen = valid && j <= pos && (window <= 0 || j > pos - window);
+        const float s = seen ? st[b][e] * sc : -INFINITY;
+        st[b][e] = s;
+        mstep = fmaxf(mstep, s);
+      }
+    mstep = group4_max(mstep);
+    const float mnew = fmaxf(mrun, mstep);
+    const float muse = mnew == -INFINITY ? 0.f : mnew;         // a query that has seen nothing yet
+    const float alpha = __builtin_amdgcn_exp2f(mrun - muse);
+    float psum = 0.f;
+    bf16x8_t phi[NC], plo[NC];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float p = __builtin_amdgcn_exp2f(st[b][e] - muse);
+        psum += p;
+        const __bf16 hi = (__bf16)p;
+        phi[b >> 1][(b & 1) * 4 + e] = hi;
+        plo[b >> 1][(b & 1) * 4 + e] = (__bf16)(p - (float)hi);
+      }
+    psum = group4_sum(psum);
+    lrun = lrun * alpha + psum;
+    mrun = mnew;
+#pragma unroll
+    for (int dt = 0; dt < CT; ++dt)
+      if (dt < ct) {
+        f32x4_t a4 = acc[dt];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a4[e] *= alpha;
+#pragma unroll
+        for (int ch = 0; ch < NC; ++ch) {
+          const uint16_t* vr = vt + (size_t)(16 * dt + r16) * VROW + 32 * ch + 4 * g;
+          const u32x2_t v0 = *reinterpret_cast<const u32x2_t*>(vr);
+          const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(vr + 16);
+          const bf16x8_t a = __builtin_bit_cast(bf16x8_t, (u32x4_t{v0.x, v0.y, v1.x, v1.y}));
+          a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, phi[ch], a4, 0, 0, 0);
+          a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, plo[ch], a4, 0, 0, 0);
+        }
+        acc[dt] = a4;
+      }
+  }
+  if (!valid) return;
+  const float inv = 1.0f / lrun;
+#pragma unroll
+  for (int dt = 0; dt < CT; ++dt)
+    if (dt < ct) {
+      u32x2_t w;
+      w.x = (unsigned)f32_to_bf16(acc[dt][0] * inv).x | ((unsigned)f32_to_bf16(acc[dt][1] * inv).x << 16);
+      w.y = (unsigned)f32_to_bf16(acc[dt][2] * inv).x | ((unsigned)f32_to_bf16(acc[dt][3] * inv).x << 16);
+      *reinterpret_cast<u32x2_t*>(out + qrow * c + 16 * dt + 4 * g) = w;
+    }
+}
+
+// Whether the kernel takes these sizes: value columns in whole tiles of 16 up to 512, rows of whole 16-byte pieces,
+// rotated columns that fit the score product's steps.
+extern "C" int gs_attention_latent_mfma_supports(int H, int c, int r) {
+  const int D = c + r;
+  if (H <= 0 || c <= 0 || r < 0 || c % 16 || D % 8) return 0;
+  if (c <= 128 && D <= 32 * (8 / 2 + 2)) return 1;
+  if (c <= 512 && D <= 32 * (32 / 2 + 2)) return 1;
+  return 0;
+}
+
+// How many consecutive tokens of a sequence one block takes (the host cuts its tile list by this).
+extern "C" int gs_attention_latent_mfma_tokens(int H) {
+  const int hb = H < LM_ROWS ? H : LM_ROWS;
+  return LM_ROWS / hb;
+}
+
+extern "C" int gs_attention_latent_mfma(const void* qa, const void* cache, const int* positions, const int* tile_seq,
+                                        const int* tile_row, const int* tile_n, int ntiles, const int* block_table,
+                                        int max_blocks, int page_size, int window, float scale, void* out, int H, int c,
+                                        int r, hipStream_t stream) {
+  GS_REQUIRE(gs_attention_latent_mfma_supports(H, c, r), "attention_latent_mfma: sizes H=%d c=%d r=%d are not taken", H, c, r);
+  GS_REQUIRE(ntiles >= 0 && page_size > 0 && max_blocks > 0 && window >= 0, "attention_latent_mfma: bad tiles/page_size/max_blocks/window");
+  GS_REQUIRE((tile_seq == nullptr) == (tile_row == nullptr) && (tile_seq == nullptr) == (tile_n == nullptr),
+             "attention_latent_mfma: a tile list has three rows");
+  if (ntiles == 0) return 0;
+  const int D = c + r, Dp = (D + 31) & ~31;
+  const int HB = H < LM_ROWS ? H : LM_ROWS;
+  const int hgroups = gs_ceil_div(H, HB);
+  GS_REQUIRE(hgroups <= 65535, "attention_latent_mfma: too many heads");
+  dim3 grid(ntiles, hgroups);
+  if (c <= 128 && D <= 32 * (8 / 2 + 2)) {
+    const size_t lds = (size_t)64 * (Dp + 8) * 2 + (size_t)c * (64 + 4) * 2;
+    attention_latent_mfma_kernel<8, 64><<<grid, 256, lds, stream>>>(
+        (const bf16*)qa, (const bf16*)cache, positions, tile_seq, tile_row, tile_n, block_table, max_blocks, page_size,
+        window, scale, (bf16*)out, H, HB, c, D);
+  } else {
+    const size_t lds = (size_t)32 * (Dp + 8) * 2 + (size_t)c * (32 + 4) * 2;
+    static bool raised = false;
+    if (!raised) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_latent_mfma_kernel<32, 32>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+      GS_REQUIRE(e == hipSuccess, "attention_latent_mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
+      raised = true;
+    }
+    GS_REQUIRE(lds <= 96 * 1024, "attention_latent_mfma: %zu bytes of LDS", lds);
+    attention_latent_mfma_kernel<32, 32><<<grid, 256, lds, stream>>>(
+        (const bf16*)qa, (const bf16*)cache, positions, tile_seq, tile_row, tile_n, block_table, max_blocks, page_size,
+        window, scale, (bf16*)out, H, HB, c, D);
+  }
+  GS_LAUNCH_CHECK("attention_latent_mfma");
+  return 0;
+}

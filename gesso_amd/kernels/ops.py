@@ -1021,3 +1021,42 @@ def moe_table(x, ids, table, up, down, shared=None, gate=None) -> torch.Tensor:
     _check(lib().gs_moe_table_down(_p(a), _dt(a), _p(ids), _p(table), top, _p(down), _dt(down), F, H, _p(shared),
                                    _p(gate) if shared is not None else None, ldg, _p(y), T, _stream()))
     return y
+
+
+def attention_latent_mfma_supports(H: int, c: int, r: int) -> bool:
+    """Whether the matrix-core kernel over latent rows takes these sizes (bfloat16; value columns in tiles of 16 up to
+    512, rows of whole 16-byte pieces)."""
+    return bool(lib().gs_attention_latent_mfma_supports(H, c, r))
+
+
+def attention_latent_mfma_tokens(H: int) -> int:
+    """How many consecutive tokens of a sequence one block of :func:`attention_latent_mfma` takes."""
+    return int(lib().gs_attention_latent_mfma_tokens(H))
+
+
+def attention_latent_mfma(qa, cache, positions, tiles, block_table, page_size, window, scale, H, c, r, ntok,
+                          out: torch.Tensor = None) -> torch.Tensor:
+    """:func:`attention_latent` on the matrix cores (bfloat16).  ``tiles``: int32 ``(3, n)``, the sequence, first row
+    and token count (at most :func:`attention_latent_mfma_tokens`) of every tile of consecutive tokens of one
+    sequence; None: sequence ``i`` brings the single token ``i``."""
+    _dev(qa, cache, positions, block_table, out, tiles)
+    _need(qa.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16, "attention_latent_mfma takes bfloat16")
+    _need(qa.shape == (ntok, H * (c + r)), "attention_latent_mfma: qa is (T, H (c + r))")
+    _need(cache.dim() == 4 and cache.shape[1:] == (1, page_size, c + r), "attention_latent_mfma: the cache is (pages, 1, page_size, c + r)")
+    _need(qa.data_ptr() % 16 == 0 and cache.data_ptr() % 16 == 0, "attention_latent_mfma: operands are 16-byte aligned")
+    _i32(positions, ntok, "positions")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (nseq, max_blocks)")
+    if tiles is None:
+        _need(block_table.shape[0] >= ntok, "attention_latent_mfma: single tokens need a block table row each")
+        n, rows = ntok, (None, None, None)
+    else:
+        _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[0] == 3, "tiles must be int32 (3, n)")
+        n, rows = tiles.shape[1], (tiles[0], tiles[1], tiles[2])
+    if out is None:
+        out = torch.empty((ntok, H * c), dtype=qa.dtype, device=qa.device)
+    _need(out.shape == (ntok, H * c) and out.dtype == qa.dtype and out.data_ptr() % 16 == 0,
+          "attention_latent_mfma: out has the wrong shape or type")
+    _check(lib().gs_attention_latent_mfma(_p(qa), _p(cache), _p(positions), _p(rows[0]), _p(rows[1]), _p(rows[2]), n,
+                                          _p(block_table), block_table.shape[1], page_size, window or 0, float(scale),
+                                          _p(out), H, c, r, _stream()))
+    return out

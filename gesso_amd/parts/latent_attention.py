@@ -98,6 +98,13 @@ class LatentAttention(Part):
     def attend(self, qa, ctx, cache) -> torch.Tensor:
         """The step's queries (absorbed form) over the cached rows: ``(T, H c)``."""
         s, ops = self.spec, self.rt.ops
+        if (qa.dtype == torch.bfloat16 and self.rt.options.latent_attention != "general"
+                and ops.attention_latent_mfma_supports(s.n_heads, s.kv_rank, s.rot_dim)):
+            # the matrix cores, whatever the step holds: tiles of consecutive tokens of one sequence, all heads of a
+            # tile in one block (a step of single tokens needs no list: sequence i is token i)
+            tiles = None if ctx.all_single else ctx.query_tiles(ops.attention_latent_mfma_tokens(s.n_heads))
+            return ops.attention_latent_mfma(qa, cache.k, ctx.positions, tiles, cache.block_table, cache.page_size,
+                                             s.window, s.scale, s.n_heads, s.kv_rank, s.rot_dim, ctx.T)
         return ops.attention_latent(qa, cache.k, ctx.positions, ctx.seq_of_token, cache.block_table, cache.page_size,
                                     s.window, s.scale, s.n_heads, s.kv_rank, s.rot_dim, ctx.T)
 

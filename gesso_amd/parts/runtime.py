@@ -41,6 +41,8 @@ class RuntimeOptions:
     ``prompt_attention``: attention of prompt portions in bfloat16: ``"wide"`` = the kernel for long portions wherever it
     takes the sizes (heads of 64), ``"tiles"`` = the kernel with tiles of 16 or 32 queries always, ``"auto"`` = the
     first for steps with a portion of at least 64 tokens, else the second.
+    ``latent_attention``: attention over cached latent rows in bfloat16: ``"auto"`` = on the matrix cores where the kernel
+    takes the sizes, ``"general"`` = the general float32-arithmetic kernel always.
     ``tiled_rows``: rows handed from one fused kernel to the next product travel in the order the matrix cores
     take them (``ops.TiledRows``): a product then loads them a contiguous kilobyte at a time.
     ``tile_weights``: keep a tile-major copy of each bfloat16 weight for the streaming kernels.
@@ -59,6 +61,7 @@ class RuntimeOptions:
     record_portions: bool = False
     tune_library: bool = False
     prompt_attention: str = "auto"
+    latent_attention: str = "auto"
     tiled_rows: bool = True
     tile_weights: bool = True
     fold_norm_rows: int = 0
@@ -69,6 +72,8 @@ class RuntimeOptions:
             raise KernelError(f"many_rows is 'auto', 'own' or 'library', not {self.many_rows!r}")
         if self.prompt_attention not in ("auto", "wide", "tiles"):
             raise KernelError(f"prompt_attention is 'auto', 'wide' or 'tiles', not {self.prompt_attention!r}")
+        if self.latent_attention not in ("auto", "general"):
+            raise KernelError(f"latent_attention is 'auto' or 'general', not {self.latent_attention!r}")
         if self.fold_norm_rows < 0 or self.weighted_rows_max < 0:
             raise KernelError("row limits are nonnegative")
 

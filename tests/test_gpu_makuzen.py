@@ -142,7 +142,7 @@ def latent_case(T, H, n, r, dv, c, seed, dtype):
                 uk=(rnd(H, n, c) / math.sqrt(c)), uv=(rnd(H, dv, c) / math.sqrt(c)))
 
 
-def attend_both(ops, case, scale, window, dtype, page_size, rows, seed=0):
+def attend_both(ops, case, scale, window, dtype, page_size, rows, seed=0, cores=False):
     """``rows``: the positions whose queries are run (one launch).  Returns the kernel's latent output mapped through
     W_uv, and the plain attention's, ``(len(rows), H, dv)`` each."""
     z, k_rot, qp, qr, uk, uv = (case[k] for k in ("z", "k_rot", "q_plain", "q_rot", "uk", "uv"))
@@ -153,9 +153,23 @@ def attend_both(ops, case, scale, window, dtype, page_size, rows, seed=0):
     want = P.windowed_attention(qp, qr, k_plain, k_rot, v, scale, window)[rows]
     qa = torch.cat([torch.einsum("thn,hnc->thc", qp, uk), qr], 2)[rows].reshape(len(rows), H * (c + r))
     pool, table = paged(torch.cat([z, k_rot], 1), page_size, -(-T // page_size) + 3, seed, dtype)
-    o = ops.attention_latent(qa.to(dtype).to(DEV), pool.to(DEV), torch.tensor(rows, dtype=torch.int32, device=DEV),
-                             torch.zeros(len(rows), dtype=torch.int32, device=DEV), table.to(DEV), page_size, window,
-                             scale, H, c, r, len(rows))
+    positions = torch.tensor(rows, dtype=torch.int32, device=DEV)
+    if cores:
+        # consecutive positions form tiles of as many tokens as a block takes; the rest are tiles of one token
+        most, tiles, at = ops.attention_latent_mfma_tokens(H), [], 0
+        while at < len(rows):
+            n = 1
+            while at + n < len(rows) and n < most and rows[at + n] == rows[at + n - 1] + 1:
+                n += 1
+            tiles.append((0, at, n))
+            at += n
+        tiles = torch.tensor(tiles, dtype=torch.int32).T.contiguous().to(DEV)
+        o = ops.attention_latent_mfma(qa.to(dtype).to(DEV), pool.to(DEV), positions, tiles, table.to(DEV), page_size,
+                                      window, scale, H, c, r, len(rows))
+    else:
+        o = ops.attention_latent(qa.to(dtype).to(DEV), pool.to(DEV), positions,
+                                 torch.zeros(len(rows), dtype=torch.int32, device=DEV), table.to(DEV), page_size, window,
+                                 scale, H, c, r, len(rows))
     got = torch.einsum("thc,hdc->thd", o.cpu().double().reshape(len(rows), H, c), uv)
     return got, want
 
@@ -171,6 +185,26 @@ def test_attention_over_latent_rows_equals_attention_over_keys_and_values(ops, d
     assert float((got - want).abs().max()) <= tol(dtype, want, 1e-5, 2e-2)
     single, _ = attend_both(ops, case, 0.3 / math.sqrt(n + r), window, dtype, ps, [T - 1])
     assert float((single[0] - want[-1]).abs().max()) <= tol(dtype, want, 1e-5, 2e-2)
+    if dtype == torch.bfloat16 and ops.attention_latent_mfma_supports(H, c, r):
+        got, _ = attend_both(ops, case, 0.3 / math.sqrt(n + r), window, dtype, ps, rows, cores=True)
+        assert float((got - want).abs().max()) <= tol(dtype, want, 1e-5, 2e-2)
+        some = [0, 1, 2, 40, 41, 97, T - 2, T - 1]
+        got, _ = attend_both(ops, case, 0.3 / math.sqrt(n + r), window, dtype, ps, some, cores=True)
+        assert float((got - want[some]).abs().max()) <= tol(dtype, want, 1e-5, 2e-2)
+
+
+@pytest.mark.parametrize("H,n,r,dv,c,window,ps", [(70, 8, 8, 8, 16, 30, 16), (16, 64, 64, 32, 512, 100, 16), (6, 32, 16, 32, 256, None, 8),
+                                                  (3, 16, 24, 8, 112, 7, 32)])
+def test_attention_over_latent_rows_on_the_matrix_cores_at_other_sizes(ops, H, n, r, dv, c, window, ps):
+    """More heads than a block takes, the widest latent, values in seven tiles, pages longer than the window."""
+    T, dtype = 200, torch.bfloat16
+    assert ops.attention_latent_mfma_supports(H, c, r)
+    case = latent_case(T, H, n, r, dv, c, 13, dtype)
+    scale = 0.3 / math.sqrt(n + r)
+    got, want = attend_both(ops, case, scale, window, dtype, ps, list(range(T)), cores=True)
+    assert float((got - want).abs().max()) <= tol(dtype, want, 1e-5, 2e-2)
+    got, _ = attend_both(ops, case, scale, window, dtype, ps, [T - 1], cores=True)
+    assert float((got[0] - want[-1]).abs().max()) <= tol(dtype, want, 1e-5, 2e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -179,7 +213,7 @@ def test_a_row_that_stands_out_is_found_far_back_at_page_borders_and_just_inside
     """One cached row is made to take nearly all of a query's weight when it is seen (its latent is the query's absorbed
     form, scaled up).  Seen: the output is that row's value.  Just outside the window: it is not.  The place is put on a
     page's last and first row, at the window's oldest place, one older than that, and (without a window) 300 back."""
-    T, H, n, r, dv, c = 340, 2, 16, 4, 8, 32
+    T, H, n, r, dv, c = 340, 2, 16, 8, 8, 32
     query = T - 1
     edge = query - window + 1 if window else None
     places = [query, query - 1, (query // ps) * ps, (query // ps) * ps - 1]
@@ -188,12 +222,13 @@ def test_a_row_that_stands_out_is_found_far_back_at_page_borders_and_just_inside
         case = latent_case(T, H, n, r, dv, c, 12, dtype)
         absorbed = torch.einsum("hn,hnc->hc", case["q_plain"][query], case["uk"])       # (H, c)
         case["z"][place] = (absorbed[0] * 40.0 / float(absorbed[0].norm())).to(dtype).double()
-        got, want = attend_both(ops, case, 1.0, window, dtype, ps, [query, query - 1, query - 5], seed=place)
         seen = window is None or place >= edge
         value = torch.einsum("dc,c->d", case["uv"][0], case["z"][place])
-        near = float((want[0, 0] - value).abs().max()) < 1e-3 * float(value.abs().max())
-        assert near == seen, (place, seen)
-        assert float((got - want).abs().max()) <= tol(dtype, want, 2e-5, 2e-2), (place, seen)
+        for cores in ([False, True] if dtype == torch.bfloat16 else [False]):
+            got, want = attend_both(ops, case, 1.0, window, dtype, ps, [query - 5, query - 1, query], seed=place, cores=cores)
+            near = float((want[2, 0] - value).abs().max()) < 1e-3 * float(value.abs().max())
+            assert near == seen, (place, seen)
+            assert float((got - want).abs().max()) <= tol(dtype, want, 2e-5, 2e-2), (place, seen, cores)
 
 
 class Tokens:
