@@ -81,6 +81,10 @@ def kv_bytes(cfg, engine, lengths) -> int:
     return kv + conv
 
 
+def vocab_of(cfg) -> int:
+    return cfg.vocab_size if hasattr(cfg, "vocab_size") else cfg.vocab
+
+
 def decode_run(engine, cfg, batch: int, prompt_len: int, steps: int, warmup: int, seed: int, temperature: float = 0.0,
                top_p: float = 1.0):
     """Prefill `batch` random prompts, then time `steps` decode steps (greedy, or with `temperature` > 0 every row
@@ -92,7 +96,7 @@ def decode_run(engine, cfg, batch: int, prompt_len: int, steps: int, warmup: int
     for rid in rids:
         engine.add_request(rid)
     from gesso_amd import StepEntry
-    prompts = [torch.randint(0, cfg.vocab_size, (prompt_len,), generator=g).tolist() for _ in rids]
+    prompts = [torch.randint(0, vocab_of(cfg), (prompt_len,), generator=g).tolist() for _ in rids]
     at = 0
     while at < batch:                                   # prompts in steps of at most 8,192 tokens
         n = max(1, min(batch - at, 8192 // prompt_len))
@@ -121,7 +125,7 @@ def decode_run(engine, cfg, batch: int, prompt_len: int, steps: int, warmup: int
 def prefill_run(engine, cfg, tokens: int, reps: int = 5):
     from gesso_amd import StepEntry
     g = torch.Generator().manual_seed(99)
-    ids = torch.randint(0, cfg.vocab_size, (tokens,), generator=g).tolist()
+    ids = torch.randint(0, vocab_of(cfg), (tokens,), generator=g).tolist()
     times = []
     warm = 4          # (a recorded step of portions is recorded at its fourth coming)
     for i in range(reps + warm):
@@ -319,6 +323,59 @@ def long_workload(seed: int = 6) -> dict:
             "data": "synthetic: uniform random token ids, random weights N(0, 0.02)"}
 
 
+MAKUZEN_SIZES = {
+    # width, layers, heads, plain / rotated / value width of a head, query and key/value rank, window, experts, used,
+    # an expert's and the shared expert's inner width, vocabulary; and the LFM2 sizes measured beside it
+    "1024": dict(width=1024, layers=8, heads=16, dim=64, rot=32, vdim=64, q_rank=384, kv_rank=256, window=1024,
+                 experts=16, top=2, ff=512, shared=1024, vocab=65536, beside="350m"),
+    "2048": dict(width=2048, layers=8, heads=16, dim=128, rot=64, vdim=128, q_rank=768, kv_rank=512, window=2048,
+                 experts=32, top=4, ff=704, shared=1408, vocab=65536, beside="1.2b"),
+}
+
+
+def makuzen_config(size: str, max_position: int = 4096):
+    from gesso_amd.config import LatentAttentionConfig, MakuzenConfig, MakuzenLayer, TableMoEConfig, YarnScaling
+    z = MAKUZEN_SIZES[size]
+    mixer = LatentAttentionConfig(heads=z["heads"], dim=z["dim"], rot_dim=z["rot"], vdim=z["vdim"], q_rank=z["q_rank"],
+                                  kv_rank=z["kv_rank"], scale=(z["dim"] + z["rot"]) ** -0.5, rot_base=1e6,
+                                  scaling=YarnScaling(4.0, 1024.0, 32.0, 1.0), window=z["window"])
+    mlp = TableMoEConfig(experts=z["experts"], top=z["top"], ff=z["ff"], shared_ff=z["shared"])
+    return MakuzenConfig(vocab=z["vocab"], width=z["width"], layers=tuple(MakuzenLayer(mixer, mlp) for _ in range(z["layers"])),
+                         embedding_scale=1.0, norm_eps=1e-5, residual_mult=0.5, max_position=max_position)
+
+
+def makuzen_workload(steps: int = 64, warmup: int = 8, sizes=("1024", "2048"), only: str = "", batches=(8, 64)) -> dict:
+    """Makuzen (latent attention over one cached row a token, table-routed experts) at two sets of layer sizes, beside
+    LFM2 of the same width and depth: a 2,048-token prompt in one step, and decode steps at 512-token prompts."""
+    import dataclasses
+    from gesso_amd import Engine
+    from gesso_amd.parts import RuntimeOptions
+    out = {"metric": "Makuzen beside LFM2 at equal width and depth: prefill and decode tok/s", "unit": "tok/s", "dtype": "bf16",
+           "data": "synthetic: uniform random token ids, random weights N(0, 0.02)", "sizes": {}}
+    for size in sizes:
+        z = MAKUZEN_SIZES[size]
+        lfm = model_config(z["beside"])
+        lfm = dataclasses.replace(lfm, num_hidden_layers=z["layers"], layer_types=lfm.layer_types[:z["layers"]])
+        row = {}
+        for name, cfg in (("makuzen", makuzen_config(size)), ("lfm2", lfm)):
+            if only and only != name:
+                continue
+            engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", page_size=16, max_context=4096,
+                                        max_tokens=max(batches) * (512 + steps + warmup + 32) + 4096, num_slots=max(batches) + 1,
+                                        options=RuntimeOptions(tune_library=True))
+            sec = prefill_run(engine, cfg, 2048)
+            r = {"prefill_tok_s": round(2048 / sec, 1), "prefill_ms": round(sec * 1e3, 3), "weights_gb": round(weight_bytes(engine) / 1e9, 3)}
+            for b in batches:
+                dt, _ = decode_run(engine, cfg, b, 512, steps, warmup, seed=40 + b)
+                r[f"decode_b{b}_tok_s"] = round(b * steps / dt, 1)
+                r[f"decode_b{b}_ms"] = round(dt / steps * 1e3, 4)
+            row[name] = r
+            del engine
+            torch.cuda.empty_cache()
+        out["sizes"][size] = row
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -338,10 +395,13 @@ def main() -> int:
     ap.add_argument("--launched-portions", action="store_true", help="launch the steps with prompt portions kernel by kernel instead of "
                     "replaying recordings of them (the prefill of the default line, --workload serve)")
     ap.add_argument("--token-budget", type=int, default=4096, help="--workload serve: the most tokens a step holds")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages", "makuzen"],
                     help="decode: the default line; serve: continuous batching at LFM2-350M sizes; long: LFM2-2.6B "
                          "sizes at a context of 32,768; gemm: the products of a 2,048-token prompt, ours beside the vendor's; "
-                         "stages: the decode step stage by stage")
+                         "stages: the decode step stage by stage; makuzen: the Makuzen design at two sets of layer sizes "
+                         "beside LFM2 of equal width and depth")
+    ap.add_argument("--makuzen-sizes", default="1024,2048", help="--workload makuzen: which of its sizes")
+    ap.add_argument("--makuzen-only", default="", choices=["", "makuzen", "lfm2"], help="--workload makuzen: one of the two models (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not measured")
@@ -349,6 +409,10 @@ def main() -> int:
     if args.workload != "decode":
         if args.workload == "stages":
             print(json.dumps(stages_workload(args.batch, min(args.steps, 32))))
+            return 0
+        if args.workload == "makuzen":
+            print(json.dumps(makuzen_workload(min(args.steps, 64), min(args.warmup, 8), tuple(args.makuzen_sizes.split(",")),
+                                              args.makuzen_only)))
             return 0
         if args.workload == "serve":
             print(json.dumps(serve_workload(record=not args.launched_portions, tune=not args.no_tune, budget=args.token_budget)))

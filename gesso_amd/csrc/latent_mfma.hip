@@ -34,7 +34,8 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
     const bf16* __restrict__ qa, const bf16* __restrict__ cache, const int* __restrict__ positions,
     const int* __restrict__ tile_seq, const int* __restrict__ tile_row, const int* __restrict__ tile_n,
     const int* __restrict__ block_table, int max_blocks, int page_size, int window, float scale,
-    bf16* __restrict__ out, int H, int HB, int c, int D) {
+    bf16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int nsplit, int rows_total, int H,
+    int HB, int c, int D) {
   constexpr int DK = CT / 2 + 2;
   constexpr int NB = KSTEP / 16, NC = KSTEP / 32, VROW = KSTEP + 4;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -54,14 +55,18 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
   const int nrows = nt * hb;
   const int pos0 = positions[row0];                  // a tile's tokens stand at consecutive positions
   const int* bt = block_table + (size_t)seq * max_blocks;
-  const int m = wave * 16 + r16;
+  // A block with at most 16 query rows (a single token of up to 16 heads): every wavefront holds the same rows and
+  // computes the same scores, and takes a quarter of the value columns.
+  const bool share = nrows <= 16;
+  const int wrow = share ? 0 : wave * 16;
+  const int m = wrow + r16;
   const bool valid = m < nrows;
   const int ti = valid ? m / hb : 0, head = h0 + (valid ? m % hb : 0);
   const int pos = pos0 + ti;
   const size_t qrow = (size_t)(row0 + ti) * H + head;
-  const bool wave_on = wave * 16 < nrows;
-  const int ti_lo = (wave * 16) / hb;
-  const int ti_hi = (wave * 16 + 15) / hb < nt - 1 ? (wave * 16 + 15) / hb : nt - 1;
+  const bool wave_on = wrow < nrows;
+  const int ti_lo = wrow / hb;
+  const int ti_hi = (wrow + 15) / hb < nt - 1 ? (wrow + 15) / hb : nt - 1;
 
   bf16x8_t qf[DK];
 #pragma unroll
@@ -79,8 +84,16 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
   const int kmax = pos0 + nt - 1;
   const int kmin = window > 0 ? (pos0 - window + 1 > 0 ? pos0 - window + 1 : 0) : 0;
   const int chunks = Dp >> 3, ct = c >> 4;
+  const int ctq = (ct + 3) >> 2;
+  const int dt_lo = share ? wave * ctq : 0;
+  const int dt_hi = share ? ((wave + 1) * ctq < ct ? (wave + 1) * ctq : ct) : ct;
+  // with the rows shared out over nsplit blocks (blockIdx.z), each takes a run of whole steps
+  const int nsteps = (kmax - kmin) / KSTEP + 1;
+  const int per = (nsteps + nsplit - 1) / nsplit;
+  const int s_begin = kmin + (int)blockIdx.z * per * KSTEP;
+  const int s_last = kmin + ((int)blockIdx.z + 1) * per * KSTEP - 1 < kmax ? kmin + ((int)blockIdx.z + 1) * per * KSTEP - 1 : kmax;
 
-  for (int s0 = kmin; s0 <= kmax; s0 += KSTEP) {
+  for (int s0 = s_begin; s0 <= s_last; s0 += KSTEP) {
     __syncthreads();
     for (int idx = tid; idx < KSTEP * chunks; idx += 256) {
       const int kk = idx / chunks, f = (idx - kk * chunks) * 8;
@@ -147,7 +160,7 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
     mrun = mnew;
 #pragma unroll
     for (int dt = 0; dt < CT; ++dt)
-      if (dt < ct) {
+      if (dt >= dt_lo && dt < dt_hi) {
         f32x4_t a4 = acc[dt];
 #pragma unroll
         for (int e = 0; e < 4; ++e) a4[e] *= alpha;
@@ -164,15 +177,51 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
       }
   }
   if (!valid) return;
+  if (nsplit > 1) {
+    // this block's share: the running maximum (base 2), the sum, and the weighted values not yet divided
+    const size_t prow = (size_t)blockIdx.z * rows_total + qrow;
+    if (g == 0 && (!share || wave == 0)) {
+      part_ml[prow * 2] = mrun;
+      part_ml[prow * 2 + 1] = lrun;
+    }
+#pragma unroll
+    for (int dt = 0; dt < CT; ++dt)
+      if (dt >= dt_lo && dt < dt_hi)
+        *reinterpret_cast<f32x4_t*>(part_o + prow * c + 16 * dt + 4 * g) = acc[dt];
+    return;
+  }
   const float inv = 1.0f / lrun;
 #pragma unroll
   for (int dt = 0; dt < CT; ++dt)
-    if (dt < ct) {
+    if (dt >= dt_lo && dt < dt_hi) {
       u32x2_t w;
       w.x = (unsigned)f32_to_bf16(acc[dt][0] * inv).x | ((unsigned)f32_to_bf16(acc[dt][1] * inv).x << 16);
       w.y = (unsigned)f32_to_bf16(acc[dt][2] * inv).x | ((unsigned)f32_to_bf16(acc[dt][3] * inv).x << 16);
       *reinterpret_cast<u32x2_t*>(out + qrow * c + 16 * dt + 4 * g) = w;
     }
+}
+
+// out[row, :] = sum_z part_o[z, row, :] 2^(m_z - M) / sum_z l_z 2^(m_z - M), M = max_z m_z: the shares of the blocks
+// that walked a row's keys in parts, added in the order of the parts.
+__global__ void attention_latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                              int nsplit, int rows_total, int c, bf16* __restrict__ out) {
+  const int row = blockIdx.x;
+  float M = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) M = fmaxf(M, part_ml[((size_t)z * rows_total + row) * 2]);
+  float L = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float* ml = part_ml + ((size_t)z * rows_total + row) * 2;
+    L += ml[1] * __builtin_amdgcn_exp2f(ml[0] - M);
+  }
+  const float inv = 1.0f / L;
+  for (int j = threadIdx.x; j < c; j += blockDim.x) {
+    float a = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const size_t prow = (size_t)z * rows_total + row;
+      a += part_o[prow * c + j] * __builtin_amdgcn_exp2f(part_ml[prow * 2] - M);
+    }
+    out[(size_t)row * c + j] = f32_to_bf16(a * inv);
+  }
 }
 
 // Whether the kernel takes these sizes: value columns in whole tiles of 16 up to 512, rows of whole 16-byte pieces,
@@ -194,22 +243,24 @@ extern "C" int gs_attention_latent_mfma_tokens(int H) {
 extern "C" int gs_attention_latent_mfma(const void* qa, const void* cache, const int* positions, const int* tile_seq,
                                         const int* tile_row, const int* tile_n, int ntiles, const int* block_table,
                                         int max_blocks, int page_size, int window, float scale, void* out, int H, int c,
-                                        int r, hipStream_t stream) {
+                                        int r, int nsplit, float* part_o, float* part_ml, int ntok, hipStream_t stream) {
   GS_REQUIRE(gs_attention_latent_mfma_supports(H, c, r), "attention_latent_mfma: sizes H=%d c=%d r=%d are not taken", H, c, r);
   GS_REQUIRE(ntiles >= 0 && page_size > 0 && max_blocks > 0 && window >= 0, "attention_latent_mfma: bad tiles/page_size/max_blocks/window");
   GS_REQUIRE((tile_seq == nullptr) == (tile_row == nullptr) && (tile_seq == nullptr) == (tile_n == nullptr),
              "attention_latent_mfma: a tile list has three rows");
+  GS_REQUIRE(nsplit >= 1 && nsplit <= 64 && (nsplit == 1 || (part_o && part_ml)), "attention_latent_mfma: %d parts need their room", nsplit);
   if (ntiles == 0) return 0;
   const int D = c + r, Dp = (D + 31) & ~31;
+  const int rows_total = ntok * H;
   const int HB = H < LM_ROWS ? H : LM_ROWS;
   const int hgroups = gs_ceil_div(H, HB);
   GS_REQUIRE(hgroups <= 65535, "attention_latent_mfma: too many heads");
-  dim3 grid(ntiles, hgroups);
+  dim3 grid(ntiles, hgroups, nsplit);
   if (c <= 128 && D <= 32 * (8 / 2 + 2)) {
     const size_t lds = (size_t)64 * (Dp + 8) * 2 + (size_t)c * (64 + 4) * 2;
     attention_latent_mfma_kernel<8, 64><<<grid, 256, lds, stream>>>(
         (const bf16*)qa, (const bf16*)cache, positions, tile_seq, tile_row, tile_n, block_table, max_blocks, page_size,
-        window, scale, (bf16*)out, H, HB, c, D);
+        window, scale, (bf16*)out, part_o, part_ml, nsplit, rows_total, H, HB, c, D);
   } else {
     const size_t lds = (size_t)32 * (Dp + 8) * 2 + (size_t)c * (32 + 4) * 2;
     static bool raised = false;
@@ -222,8 +273,12 @@ extern "C" int gs_attention_latent_mfma(const void* qa, const void* cache, const
     GS_REQUIRE(lds <= 96 * 1024, "attention_latent_mfma: %zu bytes of LDS", lds);
     attention_latent_mfma_kernel<32, 32><<<grid, 256, lds, stream>>>(
         (const bf16*)qa, (const bf16*)cache, positions, tile_seq, tile_row, tile_n, block_table, max_blocks, page_size,
-        window, scale, (bf16*)out, H, HB, c, D);
+        window, scale, (bf16*)out, part_o, part_ml, nsplit, rows_total, H, HB, c, D);
   }
   GS_LAUNCH_CHECK("attention_latent_mfma");
+  if (nsplit > 1) {
+    attention_latent_merge_kernel<<<rows_total, c >= 256 ? 256 : 64, 0, stream>>>(part_o, part_ml, nsplit, rows_total, c, (bf16*)out);
+    GS_LAUNCH_CHECK("attention_latent_merge");
+  }
   return 0;
 }

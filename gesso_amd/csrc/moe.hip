@@ -11,7 +11,7 @@
 // A wavefront computes one output at a time: its lanes walk the weight row together (contiguous loads), each lane
 // summing its columns in ascending order, then the lanes' sums are added in a fixed order; products and sums are
 // float32.  Only the chosen experts' weights are read, which is what a step of few tokens needs; steps of many tokens
-// go through the grouped product below (`moe_group_*`), which reads an expert's weights once for all of its tokens.
+// go through the grouped products of moe_group.hip, which read an expert's weights once for all of its tokens.
 #include "common.h"
 
 template <typename T, typename TW>
@@ -26,10 +26,21 @@ __global__ void moe_table_up_kernel(const T* __restrict__ x, int ldx, const int*
   const int e = table[(size_t)ids[t] * top + k];
   const TW* w = up + (size_t)e * F * H;
   T* dst = a + ((size_t)t * top + k) * F;
+  // rows of whole 16-byte pieces: eight weights a lane and load (the order of the sums depends on H alone)
+  const bool vec = (H & 7) == 0 && aligned16(w);
   for (int f = blockIdx.y * nw + wave; f < F; f += gridDim.y * nw) {
     const TW* row = w + (size_t)f * H;
     float s = 0.f;
-    for (int j = lane; j < H; j += 64) s = fmaf(to_f32(row[j]), xs[j], s);
+    if (vec) {
+      for (int j = lane * 8; j < H; j += 512) {
+        float w8[8];
+        load8f(row + j, w8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s = fmaf(w8[i], xs[j + i], s);
+      }
+    } else {
+      for (int j = lane; j < H; j += 64) s = fmaf(to_f32(row[j]), xs[j], s);
+    }
     s = wave_sum(s);
     if (lane == 0) {
       // the product is stored in the activation type before the activation, as a product of its own would be
@@ -53,13 +64,23 @@ __global__ void moe_table_down_kernel(const T* __restrict__ a, const int* __rest
   const float share = 1.0f / (float)top;
   float g = 0.f;
   if (shared) g = 1.f / (1.f + expf(-to_f32(gate[(size_t)t * ldg])));
+  const bool vec = (F & 7) == 0 && aligned16(down);
   for (int i = blockIdx.y * nw + wave; i < H; i += gridDim.y * nw) {
     float total = 0.f;
     for (int k = 0; k < top; ++k) {
       const int e = table[(size_t)ids[t] * top + k];
       const TW* row = down + ((size_t)e * H + i) * F;
       float s = 0.f;
-      for (int j = lane; j < F; j += 64) s = fmaf(to_f32(row[j]), as[k * F + j], s);
+      if (vec) {
+        for (int j = lane * 8; j < F; j += 512) {
+          float w8[8];
+          load8f(row + j, w8);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) s = fmaf(w8[u], as[k * F + j + u], s);
+        }
+      } else {
+        for (int j = lane; j < F; j += 64) s = fmaf(to_f32(row[j]), as[k * F + j], s);
+      }
       total += wave_sum(s) * share;
     }
     if (lane == 0) {

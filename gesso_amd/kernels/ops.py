@@ -1034,12 +1034,26 @@ def attention_latent_mfma_tokens(H: int) -> int:
     return int(lib().gs_attention_latent_mfma_tokens(H))
 
 
+_latent_parts = {}
+
+
+def _latent_workspace(device, rows: int, c: int, nsplit: int):
+    """Room for the shares of blocks that walk a row's keys in parts: kept per device and made anew when more is asked."""
+    need = nsplit * rows * (c + 2)
+    held = _latent_parts.get(device)
+    if held is None or held.numel() < need:
+        held = _latent_parts[device] = torch.empty(need, dtype=torch.float32, device=device)
+    return held[:nsplit * rows * c], held[nsplit * rows * c:need]
+
+
 def attention_latent_mfma(qa, cache, positions, tiles, block_table, page_size, window, scale, H, c, r, ntok,
-                          out: torch.Tensor = None) -> torch.Tensor:
+                          out: torch.Tensor = None, nsplit: int = 1) -> torch.Tensor:
     """:func:`attention_latent` on the matrix cores (bfloat16).  ``tiles``: int32 ``(3, n)``, the sequence, first row
     and token count (at most :func:`attention_latent_mfma_tokens`) of every tile of consecutive tokens of one
-    sequence; None: sequence ``i`` brings the single token ``i``."""
+    sequence; None: sequence ``i`` brings the single token ``i``.  ``nsplit`` > 1: as many blocks share a tile's keys out
+    between them in runs of whole steps, and a second kernel adds their shares."""
     _dev(qa, cache, positions, block_table, out, tiles)
+    _need(1 <= nsplit <= 64, "attention_latent_mfma: 1 to 64 parts")
     _need(qa.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16, "attention_latent_mfma takes bfloat16")
     _need(qa.shape == (ntok, H * (c + r)), "attention_latent_mfma: qa is (T, H (c + r))")
     _need(cache.dim() == 4 and cache.shape[1:] == (1, page_size, c + r), "attention_latent_mfma: the cache is (pages, 1, page_size, c + r)")
@@ -1056,7 +1070,52 @@ def attention_latent_mfma(qa, cache, positions, tiles, block_table, page_size, w
         out = torch.empty((ntok, H * c), dtype=qa.dtype, device=qa.device)
     _need(out.shape == (ntok, H * c) and out.dtype == qa.dtype and out.data_ptr() % 16 == 0,
           "attention_latent_mfma: out has the wrong shape or type")
+    part_o, part_ml = _latent_workspace(qa.device, ntok * H, c, nsplit) if nsplit > 1 else (None, None)
     _check(lib().gs_attention_latent_mfma(_p(qa), _p(cache), _p(positions), _p(rows[0]), _p(rows[1]), _p(rows[2]), n,
                                           _p(block_table), block_table.shape[1], page_size, window or 0, float(scale),
-                                          _p(out), H, c, r, _stream()))
+                                          _p(out), H, c, r, nsplit, _p(part_o), _p(part_ml), ntok, _stream()))
     return out
+
+
+def moe_grouped_ok(x, up, down) -> bool:
+    """Whether :func:`moe_table_grouped` takes these operands: bfloat16 throughout, widths in whole 16-byte pieces."""
+    bf = torch.bfloat16
+    return (x.dtype is bf and up.dtype is bf and down.dtype is bf and x.dim() == 2 and x.stride(1) == 1
+            and x.shape[1] % 8 == 0 and up.shape[1] % 8 == 0 and (x.shape[0] <= 1 or x.stride(0) % 8 == 0)
+            and x.data_ptr() % 16 == 0 and up.shape[0] <= 4096)
+
+
+def moe_table_grouped(x, ids, table, up, down, shared=None, gate=None) -> torch.Tensor:
+    """:func:`moe_table` for steps of many tokens (bfloat16): the (token, choice) pairs are sorted by expert on the
+    device and every expert's weights are read once, by products on the matrix cores over its pairs' rows."""
+    _dev(ids, table, up, down, shared)
+    _need(moe_grouped_ok(x, up, down), "moe_table_grouped: bfloat16 rows and weights, widths multiples of 8")
+    T, H = x.shape
+    E, F, Hw = up.shape
+    _need(Hw == H and down.shape == (E, H, F), "moe_table_grouped: up is (E, F, H), down (E, H, F)")
+    _need(table.dtype == torch.int32 and table.dim() == 2, "moe_table_grouped: the table is int32 (vocab, top)")
+    top = table.shape[1]
+    _i32(ids, T, "token ids")
+    ldg = 0
+    if shared is not None:
+        _need(shared.shape == (T, H) and shared.dtype == x.dtype and gate is not None and gate.is_cuda and gate.dim() == 2
+              and gate.shape[0] == T and gate.dtype == x.dtype and gate.stride(1) == 1,
+              "moe_table_grouped: shared rows (T, H) come with a gate (T, >= 1) of the rows' type")
+        ldg = gate.stride(0) if T > 1 else gate.shape[1]
+    P = T * top
+    dev = x.device
+    max_tiles = -(-P // lib().gs_moe_group_rows()) + E
+    index = torch.empty(2 * P + 3 * max_tiles + 1, dtype=torch.int32, device=dev)
+    perm, place_of, tiles, n_tiles = index[:P], index[P:2 * P], index[2 * P:2 * P + 3 * max_tiles], index[2 * P + 3 * max_tiles:]
+    inner = torch.empty((P, F), dtype=torch.bfloat16, device=dev)
+    ys = torch.empty((P, H), dtype=torch.float32, device=dev)
+    y = torch.empty((T, H), dtype=x.dtype, device=dev)
+    s = _stream()
+    L = lib()
+    _check(L.gs_moe_route(_p(ids), _p(table), T, top, E, _p(perm), _p(place_of), _p(tiles), max_tiles, _p(n_tiles), s))
+    _check(L.gs_moe_group_gemm(_p(x), x.stride(0) if T > 1 else H, _p(perm), _p(up), _p(inner), BF16, F, _p(tiles), max_tiles,
+                               _p(n_tiles), F, H, 2, s))
+    _check(L.gs_moe_group_gemm(_p(inner), F, None, _p(down), _p(ys), F32, H, _p(tiles), max_tiles, _p(n_tiles), H, F, 0, s))
+    _check(L.gs_moe_combine(_p(ys), _p(place_of), top, _p(shared), _p(gate) if shared is not None else None, ldg, _p(y),
+                            _dt(y), T, H, s))
+    return y

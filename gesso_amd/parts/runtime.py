@@ -43,6 +43,8 @@ class RuntimeOptions:
     first for steps with a portion of at least 64 tokens, else the second.
     ``latent_attention``: attention over cached latent rows in bfloat16: ``"auto"`` = on the matrix cores where the kernel
     takes the sizes, ``"general"`` = the general float32-arithmetic kernel always.
+    ``routed_experts``: a table-routed mixture of experts in bfloat16: ``"auto"`` = pairs sorted by expert and products on
+    the matrix cores once a step's (token, choice) pairs outnumber the experts twice over, ``"token"`` = token by token always.
     ``tiled_rows``: rows handed from one fused kernel to the next product travel in the order the matrix cores
     take them (``ops.TiledRows``): a product then loads them a contiguous kilobyte at a time.
     ``tile_weights``: keep a tile-major copy of each bfloat16 weight for the streaming kernels.
@@ -62,6 +64,7 @@ class RuntimeOptions:
     tune_library: bool = False
     prompt_attention: str = "auto"
     latent_attention: str = "auto"
+    routed_experts: str = "auto"
     tiled_rows: bool = True
     tile_weights: bool = True
     fold_norm_rows: int = 0
@@ -74,6 +77,8 @@ class RuntimeOptions:
             raise KernelError(f"prompt_attention is 'auto', 'wide' or 'tiles', not {self.prompt_attention!r}")
         if self.latent_attention not in ("auto", "general"):
             raise KernelError(f"latent_attention is 'auto' or 'general', not {self.latent_attention!r}")
+        if self.routed_experts not in ("auto", "token"):
+            raise KernelError(f"routed_experts is 'auto' or 'token', not {self.routed_experts!r}")
         if self.fold_norm_rows < 0 or self.weighted_rows_max < 0:
             raise KernelError("row limits are nonnegative")
 

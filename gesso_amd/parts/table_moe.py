@@ -67,6 +67,11 @@ class TableMoE(Part):
         if shared is not None and gate is None:
             # an ungated shared expert: sigmoid(large) = 1
             gate = torch.full((x.shape[0], 1), 80.0, dtype=x.dtype, device=x.device)
+        # once the pairs outnumber the experts twice over, sorting them by expert reads less: each expert's weights
+        # once, instead of once a pair (the option "token" keeps the token-by-token kernels for every step)
+        if (x.shape[0] * s.top >= 2 * s.n_experts and rt.options.routed_experts != "token"
+                and ops.moe_grouped_ok(x, self.up, self.down)):
+            return ops.moe_table_grouped(x, ctx.token_ids, self.table, self.up, self.down, shared=shared, gate=gate)
         return ops.moe_table(x, ctx.token_ids, self.table, self.up, self.down, shared=shared, gate=gate)
 
 
