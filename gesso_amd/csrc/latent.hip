@@ -9,8 +9,8 @@
 //   latent_prep       per token: RMS norm of the query latent -> rows for the query product; RMS norm of the
 //                     key/value latent, rotation of the shared key features, both into the token's cache row
 //   latent_q_rot      rotates the rotated part of every head's query into its place behind the absorbed part
-//   heads_product     Y[t, h, :] = W[h] X[t, h, :] for all heads in one launch (float32 FMAs, fixed summation order),
-//                     with an optional gate: times sigmoid(G[t, h])
+//   heads_product     Y[t, h, :] = W[h] X[t, h, :] for all heads in one launch, with an optional gate: times
+//                     sigmoid(G[t, h]); float32 FMAs in a fixed summation order, or the matrix cores for bfloat16
 //   attention_latent  the general attention kernel over such rows: any sizes, float32 arithmetic
 //
 // All norms, angles, scores, softmax weights and the gate's sigmoid are float32.
@@ -184,6 +184,67 @@ __global__ void heads_product_kernel(const TX* __restrict__ X, int ldx, int hx, 
   }
 }
 
+// The same product on the matrix cores (bfloat16 rows and weights, float32 sums): v_mfma_f32_16x16x32_bf16 with both
+// operands loaded straight from memory in operand order (lane l: row or weight row l % 16, eight consecutive k at
+// 8 (l / 16)); a head's weight is small and stays in the caches, so nothing is staged.  A wavefront owns 16 rows x
+// 16 NTW columns of one head; the four wavefronts of a block own four such pieces, and no barrier is needed.
+typedef __attribute__((ext_vector_type(8))) __bf16 hp_bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float hp_f32x4_t;
+typedef __attribute__((ext_vector_type(4))) unsigned hp_u32x4_t;
+
+template <int NTW>
+__global__ __launch_bounds__(256) void heads_product_mfma_kernel(const bf16* __restrict__ X, int ldx, int hx,
+                                                                 const bf16* __restrict__ W, bf16* __restrict__ Y,
+                                                                 int ldy, int hy, const bf16* __restrict__ G, int ldg,
+                                                                 int M, int N, int K) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
+  const int h = blockIdx.y;
+  const int mtiles = (M + 15) >> 4, ngroups = (N + 16 * NTW - 1) / (16 * NTW);
+  const int item = blockIdx.x * 4 + wave;
+  if (item >= mtiles * ngroups) return;
+  const int m0 = (item % mtiles) * 16, n0 = (item / mtiles) * 16 * NTW;
+  const int mrow = m0 + r16 < M ? m0 + r16 : M - 1;
+  const bf16* xp = X + (size_t)mrow * ldx + (size_t)h * hx + 8 * g;
+  const bf16* wp[NTW];
+#pragma unroll
+  for (int j = 0; j < NTW; ++j) {
+    const int n = n0 + 16 * j + r16 < N ? n0 + 16 * j + r16 : N - 1;
+    wp[j] = W + ((size_t)h * N + n) * K + 8 * g;
+  }
+  hp_f32x4_t acc[NTW];
+#pragma unroll
+  for (int j = 0; j < NTW; ++j) acc[j] = hp_f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool in = k0 + 8 * g < K;                      // K in whole pieces of 8: a piece is inside or outside
+    const int kk = in ? k0 : -8 * g;
+    hp_u32x4_t a = *reinterpret_cast<const hp_u32x4_t*>(xp + kk);
+    a = in ? a : hp_u32x4_t{0u, 0u, 0u, 0u};
+    hp_u32x4_t b[NTW];
+#pragma unroll
+    for (int j = 0; j < NTW; ++j) {
+      b[j] = *reinterpret_cast<const hp_u32x4_t*>(wp[j] + kk);
+      b[j] = in ? b[j] : hp_u32x4_t{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int j = 0; j < NTW; ++j)
+      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(hp_bf16x8_t, a), __builtin_bit_cast(hp_bf16x8_t, b[j]),
+                                                       acc[j], 0, 0, 0);
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int m = m0 + 4 * g + e;
+    if (m >= M) continue;
+    float gate = 1.f;
+    if (G) gate = 1.f / (1.f + expf(-to_f32(G[(size_t)m * ldg + h])));
+#pragma unroll
+    for (int j = 0; j < NTW; ++j) {
+      const int n = n0 + 16 * j + r16;
+      if (n < N) Y[(size_t)m * ldy + (size_t)h * hy + n] = f32_to_bf16(acc[j][e] * gate);
+    }
+  }
+}
+
 extern "C" int gs_heads_product(const void* X, int x_dtype, int ldx, int hx, const void* W, int w_dtype, void* Y,
                                 int ldy, int hy, const void* G, int ldg, int M, int N, int K, int H,
                                 hipStream_t stream) {
@@ -193,6 +254,23 @@ extern "C" int gs_heads_product(const void* X, int x_dtype, int ldx, int hx, con
              "heads_product: heads reach past their rows (ldx=%d hx=%d K=%d, ldy=%d hy=%d N=%d)", ldx, hx, K, ldy, hy, N);
   GS_REQUIRE(G == nullptr || ldg >= H, "heads_product: gate rows of %d hold no %d heads", ldg, H);
   if (M == 0) return 0;
+  if (x_dtype == GS_BF16 && w_dtype == GS_BF16 && K % 8 == 0 && ldx % 8 == 0 && hx % 8 == 0 && ((uintptr_t)X & 15) == 0 &&
+      ((uintptr_t)W & 15) == 0) {
+    const int mtiles = gs_ceil_div(M, 16);
+    // few rows: narrow pieces, so that a head's weight is spread over more wavefronts
+    const int ntw = M <= 64 ? 1 : 4;
+    const long items = (long)mtiles * gs_ceil_div(N, 16 * ntw);
+    GS_REQUIRE(items / 4 + 1 < (1L << 31), "heads_product: too many tiles");
+    dim3 grid((unsigned)gs_ceil_div(items, 4), H);
+    if (ntw == 1)
+      heads_product_mfma_kernel<1><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, hx, (const bf16*)W, (bf16*)Y, ldy, hy,
+                                                            (const bf16*)G, ldg, M, N, K);
+    else
+      heads_product_mfma_kernel<4><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, hx, (const bf16*)W, (bf16*)Y, ldy, hy,
+                                                            (const bf16*)G, ldg, M, N, K);
+    GS_LAUNCH_CHECK("heads_product_mfma");
+    return 0;
+  }
   dim3 grid(gs_ceil_div(N, HP_TN), gs_ceil_div(M, HP_TM), H);
   if (x_dtype == GS_F32 && w_dtype == GS_F32)
     heads_product_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)X, ldx, hx, (const float*)W, (float*)Y,

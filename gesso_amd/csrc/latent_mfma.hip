@@ -93,27 +93,47 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
   const int s_begin = kmin + (int)blockIdx.z * per * KSTEP;
   const int s_last = kmin + ((int)blockIdx.z + 1) * per * KSTEP - 1 < kmax ? kmin + ((int)blockIdx.z + 1) * per * KSTEP - 1 : kmax;
 
+  // This thread's pieces of a step's rows: piece i is 16 bytes at column pf[i] of row pk[i] of the step (pk < 0: none).
+  // A step's pieces are asked for while the step before it is computed, all of them before any is waited for, and go
+  // into LDS after that step's products: row-major for the scores, and their value columns transposed.
+  constexpr int NL = KSTEP * (DK * 4) / 256;
+  int pk[NL], pf[NL];
+#pragma unroll
+  for (int i = 0; i < NL; ++i) {
+    const int idx = tid + 256 * i;
+    pk[i] = idx < KSTEP * chunks ? idx / chunks : -1;
+    pf[i] = (idx - (idx / chunks) * chunks) * 8;
+  }
+  u32x4_t pv[NL];
+#define LM_ASK(s0)                                                                                              \
+  {                                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < NL; ++i) {                                                            \
+      const int j = (s0) + pk[i];                                                                               \
+      pv[i] = u32x4_t{0u, 0u, 0u, 0u};                                                                          \
+      if (pk[i] >= 0 && j <= kmax && pf[i] < D) {                                                               \
+        const int page = bt[j / page_size];                                                                     \
+        pv[i] = *reinterpret_cast<const u32x4_t*>(cache + ((size_t)page * page_size + j % page_size) * D + pf[i]); \
+      }                                                                                                         \
+    }                                                                                                           \
+  }
+  if (s_begin <= s_last) LM_ASK(s_begin);
   for (int s0 = s_begin; s0 <= s_last; s0 += KSTEP) {
     __syncthreads();
-    for (int idx = tid; idx < KSTEP * chunks; idx += 256) {
-      const int kk = idx / chunks, f = (idx - kk * chunks) * 8;
-      const int j = s0 + kk;
-      u32x4_t v = {0u, 0u, 0u, 0u};
-      if (j <= kmax && f < D) {
-        const int page = bt[j / page_size];
-        v = *reinterpret_cast<const u32x4_t*>(cache + ((size_t)page * page_size + j % page_size) * D + f);
-      }
-      *reinterpret_cast<u32x4_t*>(ks + (size_t)kk * krow + f) = v;
-      if (f < c) {
-        const unsigned w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          vt[(size_t)(f + 2 * e) * VROW + kk] = (uint16_t)(w[e] & 0xffffu);
-          vt[(size_t)(f + 2 * e + 1) * VROW + kk] = (uint16_t)(w[e] >> 16);
+    for (int i = 0; i < NL; ++i)
+      if (pk[i] >= 0) {
+        *reinterpret_cast<u32x4_t*>(ks + (size_t)pk[i] * krow + pf[i]) = pv[i];
+        if (pf[i] < c) {
+          const unsigned w[4] = {pv[i].x, pv[i].y, pv[i].z, pv[i].w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            vt[(size_t)(pf[i] + 2 * e) * VROW + pk[i]] = (uint16_t)(w[e] & 0xffffu);
+            vt[(size_t)(pf[i] + 2 * e + 1) * VROW + pk[i]] = (uint16_t)(w[e] >> 16);
+          }
         }
       }
-    }
     __syncthreads();
+    if (s0 + KSTEP <= s_last) LM_ASK(s0 + KSTEP);
     // a wavefront none of whose queries sees a row of this step waits for the next
     const bool step_on = wave_on && s0 <= pos0 + ti_hi && (window <= 0 || s0 + KSTEP - 1 > pos0 + ti_lo - window);
     if (!step_on) continue;

@@ -118,9 +118,10 @@ def test_latent_q_rot_puts_the_rotated_part_behind_the_absorbed_one(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,H,N,K", [(1, 3, 48, 24), (70, 5, 20, 36), (130, 2, 64, 130), (9, 1, 7, 3)])
+@pytest.mark.parametrize("M,H,N,K", [(1, 3, 48, 24), (70, 5, 20, 36), (130, 2, 64, 130), (9, 1, 7, 3), (8, 4, 64, 32),
+                                     (200, 3, 40, 72), (33, 2, 16, 8), (64, 16, 512, 128), (65, 2, 128, 512)])
 def test_heads_product_with_and_without_gate(ops, dtype, M, H, N, K):
-    x = torch.randn(M, H * K + 3, generator=gen(8)).to(dtype)
+    x = torch.randn(M, H * K + 8, generator=gen(8)).to(dtype)      # (rows of whole 16-byte pieces where H K allows)
     w = (torch.randn(H, N, K, generator=gen(9)) / math.sqrt(K)).to(dtype)
     g = torch.randn(M, H + 2, generator=gen(10)).to(dtype)
     for gate in (None, g):
