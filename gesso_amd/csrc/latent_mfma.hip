@@ -96,13 +96,17 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
   // This thread's pieces of a step's rows: piece i is 16 bytes at column pf[i] of row pk[i] of the step (pk < 0: none).
   // A step's pieces are asked for while the step before it is computed, all of them before any is waited for, and go
   // into LDS after that step's products: row-major for the scores, and their value columns transposed.
+  // Of a wavefront's 64 pieces sixteen rows have four neighbouring pieces each: 64 contiguous bytes a row from memory,
+  // and the transposed 2-byte stores of one instruction fall into different LDS banks (sixteen neighbouring rows of
+  // one column are eight words; the four columns groups lie 16 banks apart).
   constexpr int NL = KSTEP * (DK * 4) / 256;
   int pk[NL], pf[NL];
 #pragma unroll
   for (int i = 0; i < NL; ++i) {
-    const int idx = tid + 256 * i;
-    pk[i] = idx < KSTEP * chunks ? idx / chunks : -1;
-    pf[i] = (idx - (idx / chunks) * chunks) * 8;
+    const int idx = tid + 256 * i, unit = idx >> 6, l = idx & 63;
+    const int kk = (unit % (KSTEP / 16)) * 16 + (l & 15), ch = (unit / (KSTEP / 16)) * 4 + (l >> 4);
+    pk[i] = ch < chunks ? kk : -1;
+    pf[i] = ch * 8;
   }
   u32x4_t pv[NL];
 #define LM_ASK(s0)                                                                                              \
