@@ -93,31 +93,38 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
   const int s_begin = kmin + (int)blockIdx.z * per * KSTEP;
   const int s_last = kmin + ((int)blockIdx.z + 1) * per * KSTEP - 1 < kmax ? kmin + ((int)blockIdx.z + 1) * per * KSTEP - 1 : kmax;
 
-  // This thread's pieces of a step's rows: piece i is 16 bytes at column pf[i] of row pk[i] of the step (pk < 0: none).
-  // A step's pieces are asked for while the step before it is computed, all of them before any is waited for, and go
-  // into LDS after that step's products: row-major for the scores, and their value columns transposed.
-  // Of a wavefront's 64 pieces sixteen rows have four neighbouring pieces each: 64 contiguous bytes a row from memory,
-  // and the transposed 2-byte stores of one instruction fall into different LDS banks (sixteen neighbouring rows of
-  // one column are eight words; the four columns groups lie 16 banks apart).
+  // This thread's pieces of a step's rows: 16 bytes each.  A step's pieces are asked for while the step before it is
+  // computed, all of them before any is waited for, and go into LDS after that step's products: row-major for the
+  // scores, and their value columns transposed.  Of a wavefront's 64 pieces sixteen rows have four neighbouring pieces
+  // each: 64 contiguous bytes a row from memory, and the transposed 2-byte stores of one instruction fall into
+  // different LDS banks (sixteen neighbouring rows of one column are eight words; the four column groups lie 16 banks
+  // apart).
+  // All pieces of a thread belong to one row of the step (its pieces lie whole wavefronts of four apart, and the rows
+  // repeat every KSTEP / 16 wavefronts), so a step costs a thread one page lookup; where a piece goes in LDS is the
+  // same in every step.
   constexpr int NL = KSTEP * (DK * 4) / 256;
-  int pk[NL], pf[NL];
+  const int pk = ((tid >> 6) % (KSTEP / 16)) * 16 + (lane & 15);       // this thread's row of a step
+  int pf[NL];                                                         // its pieces' columns (< 0: none)
+  bf16* ksp[NL];
+  uint16_t* vtp[NL];
 #pragma unroll
   for (int i = 0; i < NL; ++i) {
-    const int idx = tid + 256 * i, unit = idx >> 6, l = idx & 63;
-    const int kk = (unit % (KSTEP / 16)) * 16 + (l & 15), ch = (unit / (KSTEP / 16)) * 4 + (l >> 4);
-    pk[i] = ch < chunks ? kk : -1;
-    pf[i] = ch * 8;
+    const int unit = (tid >> 6) + 4 * i;
+    const int ch = (unit / (KSTEP / 16)) * 4 + (lane >> 4);
+    pf[i] = ch < chunks ? ch * 8 : -1;
+    ksp[i] = ks + (size_t)pk * krow + ch * 8;
+    vtp[i] = vt + (size_t)ch * 8 * VROW + pk;
   }
   u32x4_t pv[NL];
 #define LM_ASK(s0)                                                                                              \
   {                                                                                                             \
+    const int j = (s0) + pk;                                                                                    \
+    const bool row_in = j <= kmax;                                                                              \
+    const int jj = row_in ? j : kmax;                                                                           \
+    const bf16* src = cache + ((size_t)bt[jj / page_size] * page_size + jj % page_size) * D;                    \
     _Pragma("unroll") for (int i = 0; i < NL; ++i) {                                                            \
-      const int j = (s0) + pk[i];                                                                               \
       pv[i] = u32x4_t{0u, 0u, 0u, 0u};                                                                          \
-      if (pk[i] >= 0 && j <= kmax && pf[i] < D) {                                                               \
-        const int page = bt[j / page_size];                                                                     \
-        pv[i] = *reinterpret_cast<const u32x4_t*>(cache + ((size_t)page * page_size + j % page_size) * D + pf[i]); \
-      }                                                                                                         \
+      if (row_in && pf[i] >= 0 && pf[i] < D) pv[i] = *reinterpret_cast<const u32x4_t*>(src + pf[i]);            \
     }                                                                                                           \
   }
   if (s_begin <= s_last) LM_ASK(s_begin);
@@ -125,14 +132,14 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < NL; ++i)
-      if (pk[i] >= 0) {
-        *reinterpret_cast<u32x4_t*>(ks + (size_t)pk[i] * krow + pf[i]) = pv[i];
+      if (pf[i] >= 0) {
+        *reinterpret_cast<u32x4_t*>(ksp[i]) = pv[i];
         if (pf[i] < c) {
           const unsigned w[4] = {pv[i].x, pv[i].y, pv[i].z, pv[i].w};
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            vt[(size_t)(pf[i] + 2 * e) * VROW + pk[i]] = (uint16_t)(w[e] & 0xffffu);
-            vt[(size_t)(pf[i] + 2 * e + 1) * VROW + pk[i]] = (uint16_t)(w[e] >> 16);
+            vtp[i][(2 * e) * VROW] = (uint16_t)(w[e] & 0xffffu);
+            vtp[i][(2 * e + 1) * VROW] = (uint16_t)(w[e] >> 16);
           }
         }
       }
