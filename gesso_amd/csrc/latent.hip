@@ -186,40 +186,50 @@ __global__ void heads_product_kernel(const TX* __restrict__ X, int ldx, int hx, 
 
 // The same product on the matrix cores (bfloat16 rows and weights, float32 sums): v_mfma_f32_16x16x32_bf16 with both
 // operands loaded straight from memory in operand order (lane l: row or weight row l % 16, eight consecutive k at
-// 8 (l / 16)); a head's weight is small and stays in the caches, so nothing is staged.  A wavefront owns 16 rows x
+// 8 (l / 16)); a head's weight is small and stays in the caches, so nothing is staged.  A wavefront owns 16 MTW rows x
 // 16 NTW columns of one head; the four wavefronts of a block own four such pieces, and no barrier is needed.
 typedef __attribute__((ext_vector_type(8))) __bf16 hp_bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float hp_f32x4_t;
 typedef __attribute__((ext_vector_type(4))) unsigned hp_u32x4_t;
 
-template <int NTW>
+template <int NTW, int MTW>
 __global__ __launch_bounds__(256) void heads_product_mfma_kernel(const bf16* __restrict__ X, int ldx, int hx,
                                                                  const bf16* __restrict__ W, bf16* __restrict__ Y,
                                                                  int ldy, int hy, const bf16* __restrict__ G, int ldg,
                                                                  int M, int N, int K) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
   const int h = blockIdx.y;
-  const int mtiles = (M + 15) >> 4, ngroups = (N + 16 * NTW - 1) / (16 * NTW);
+  const int mtiles = (M + 16 * MTW - 1) / (16 * MTW), ngroups = (N + 16 * NTW - 1) / (16 * NTW);
   const int item = blockIdx.x * 4 + wave;
   if (item >= mtiles * ngroups) return;
-  const int m0 = (item % mtiles) * 16, n0 = (item / mtiles) * 16 * NTW;
-  const int mrow = m0 + r16 < M ? m0 + r16 : M - 1;
-  const bf16* xp = X + (size_t)mrow * ldx + (size_t)h * hx + 8 * g;
+  const int m0 = (item % mtiles) * 16 * MTW, n0 = (item / mtiles) * 16 * NTW;
+  const bf16* xp[MTW];
+#pragma unroll
+  for (int i = 0; i < MTW; ++i) {
+    const int mrow = m0 + 16 * i + r16 < M ? m0 + 16 * i + r16 : M - 1;
+    xp[i] = X + (size_t)mrow * ldx + (size_t)h * hx + 8 * g;
+  }
   const bf16* wp[NTW];
 #pragma unroll
   for (int j = 0; j < NTW; ++j) {
     const int n = n0 + 16 * j + r16 < N ? n0 + 16 * j + r16 : N - 1;
     wp[j] = W + ((size_t)h * N + n) * K + 8 * g;
   }
-  hp_f32x4_t acc[NTW];
+  hp_f32x4_t acc[MTW][NTW];
 #pragma unroll
-  for (int j = 0; j < NTW; ++j) acc[j] = hp_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < MTW; ++i)
+#pragma unroll
+    for (int j = 0; j < NTW; ++j) acc[i][j] = hp_f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 4
   for (int k0 = 0; k0 < K; k0 += 32) {
     const bool in = k0 + 8 * g < K;                      // K in whole pieces of 8: a piece is inside or outside
     const int kk = in ? k0 : -8 * g;
-    hp_u32x4_t a = *reinterpret_cast<const hp_u32x4_t*>(xp + kk);
-    a = in ? a : hp_u32x4_t{0u, 0u, 0u, 0u};
+    hp_u32x4_t a[MTW];
+#pragma unroll
+    for (int i = 0; i < MTW; ++i) {
+      a[i] = *reinterpret_cast<const hp_u32x4_t*>(xp[i] + kk);
+      a[i] = in ? a[i] : hp_u32x4_t{0u, 0u, 0u, 0u};
+    }
     hp_u32x4_t b[NTW];
 #pragma unroll
     for (int j = 0; j < NTW; ++j) {
@@ -227,22 +237,26 @@ __global__ __launch_bounds__(256) void heads_product_mfma_kernel(const bf16* __r
       b[j] = in ? b[j] : hp_u32x4_t{0u, 0u, 0u, 0u};
     }
 #pragma unroll
-    for (int j = 0; j < NTW; ++j)
-      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(hp_bf16x8_t, a), __builtin_bit_cast(hp_bf16x8_t, b[j]),
-                                                       acc[j], 0, 0, 0);
+    for (int i = 0; i < MTW; ++i)
+#pragma unroll
+      for (int j = 0; j < NTW; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(hp_bf16x8_t, a[i]),
+                                                            __builtin_bit_cast(hp_bf16x8_t, b[j]), acc[i][j], 0, 0, 0);
   }
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const int m = m0 + 4 * g + e;
-    if (m >= M) continue;
-    float gate = 1.f;
-    if (G) gate = 1.f / (1.f + expf(-to_f32(G[(size_t)m * ldg + h])));
+  for (int i = 0; i < MTW; ++i)
 #pragma unroll
-    for (int j = 0; j < NTW; ++j) {
-      const int n = n0 + 16 * j + r16;
-      if (n < N) Y[(size_t)m * ldy + (size_t)h * hy + n] = f32_to_bf16(acc[j][e] * gate);
+    for (int e = 0; e < 4; ++e) {
+      const int m = m0 + 16 * i + 4 * g + e;
+      if (m >= M) continue;
+      float gate = 1.f;
+      if (G) gate = 1.f / (1.f + expf(-to_f32(G[(size_t)m * ldg + h])));
+#pragma unroll
+      for (int j = 0; j < NTW; ++j) {
+        const int n = n0 + 16 * j + r16;
+        if (n < N) Y[(size_t)m * ldy + (size_t)h * hy + n] = f32_to_bf16(acc[i][j][e] * gate);
+      }
     }
-  }
 }
 
 extern "C" int gs_heads_product(const void* X, int x_dtype, int ldx, int hx, const void* W, int w_dtype, void* Y,
@@ -256,17 +270,17 @@ extern "C" int gs_heads_product(const void* X, int x_dtype, int ldx, int hx, con
   if (M == 0) return 0;
   if (x_dtype == GS_BF16 && w_dtype == GS_BF16 && K % 8 == 0 && ldx % 8 == 0 && hx % 8 == 0 && ((uintptr_t)X & 15) == 0 &&
       ((uintptr_t)W & 15) == 0) {
-    const int mtiles = gs_ceil_div(M, 16);
-    // few rows: narrow pieces, so that a head's weight is spread over more wavefronts
-    const int ntw = M <= 64 ? 1 : 4;
+    // few rows: narrow pieces, so that a head's weight is spread over more wavefronts; many: 32 x 64 a wavefront
+    const int ntw = M <= 64 ? 1 : 4, mtw = M <= 64 ? 1 : 2;
+    const int mtiles = gs_ceil_div(M, 16 * mtw);
     const long items = (long)mtiles * gs_ceil_div(N, 16 * ntw);
     GS_REQUIRE(items / 4 + 1 < (1L << 31), "heads_product: too many tiles");
     dim3 grid((unsigned)gs_ceil_div(items, 4), H);
     if (ntw == 1)
-      heads_product_mfma_kernel<1><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, hx, (const bf16*)W, (bf16*)Y, ldy, hy,
+      heads_product_mfma_kernel<1, 1><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, hx, (const bf16*)W, (bf16*)Y, ldy, hy,
                                                             (const bf16*)G, ldg, M, N, K);
     else
-      heads_product_mfma_kernel<4><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, hx, (const bf16*)W, (bf16*)Y, ldy, hy,
+      heads_product_mfma_kernel<4, 2><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, hx, (const bf16*)W, (bf16*)Y, ldy, hy,
                                                             (const bf16*)G, ldg, M, N, K);
     GS_LAUNCH_CHECK("heads_product_mfma");
     return 0;

@@ -106,13 +106,13 @@ class LatentAttention(Part):
             nsplit = 1
             if ctx.all_single:
                 # single tokens: few blocks, each with a long walk; the keys are shared out over blocks until the chip
-                # is full, a part at least 128 keys long (the bound on the keys is the longest sequence's, or what the
+                # is full, a part at least 64 keys long (the bound on the keys is the longest sequence's, or what the
                 # block tables hold where the host does not know it, cut by the window)
                 longest = ctx.max_kv_len if ctx.max_kv_len is not None else cache.block_table.shape[1] * cache.page_size
                 if s.window:
                     longest = min(longest, s.window)
                 blocks = ctx.T * -(-s.n_heads // 64)
-                nsplit = max(1, min(longest // 128, 64, self.rt.compute_units // max(1, blocks)))
+                nsplit = max(1, min(longest // 64, 64, self.rt.compute_units // max(1, blocks)))
             return ops.attention_latent_mfma(qa, cache.k, ctx.positions, tiles, cache.block_table, cache.page_size,
                                              s.window, s.scale, s.n_heads, s.kv_rank, s.rot_dim, ctx.T, nsplit=nsplit)
         return ops.attention_latent(qa, cache.k, ctx.positions, ctx.seq_of_token, cache.block_table, cache.page_size,
