@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int Dp = (D + 31) & ~31, krow = Dp + 8;
   bf16* ks = reinterpret_cast<bf16*>(lds);                                            // [KSTEP][krow]
-  uint16_t* vt = reinterpret_cast<uint16_t*>(lds + (size_t)KSTEP * krow * 2);         // [c][VROW]
+  uint16_t* vt = reinterpret_cast<uint16_t*>(lds + (size_t)KSTEP * krow * 2);         // [c up to whole 64][VROW]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r16 = lane & 15, g = lane >> 4;
   const int tile = blockIdx.x;
   int seq = tile, row0 = tile, nt = 1;               // without a list: sequence i brings the single token i
@@ -84,9 +84,12 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
   const int kmax = pos0 + nt - 1;
   const int kmin = window > 0 ? (pos0 - window + 1 > 0 ? pos0 - window + 1 : 0) : 0;
   const int chunks = Dp >> 3, ct = c >> 4;
-  const int ctq = (ct + 3) >> 2;
-  const int dt_lo = share ? wave * ctq : 0;
-  const int dt_hi = share ? ((wave + 1) * ctq < ct ? (wave + 1) * ctq : ct) : ct;
+  // value tiles go in groups of four (a last group may reach past c: its spare tiles are computed on LDS rows that
+  // belong to nobody and never stored); with shared rows a wavefront takes a quarter of the groups
+  const int ngr = (ct + 3) >> 2, gq = (ngr + 3) >> 2;
+  const int g_lo = share ? wave * gq : 0;
+  const int g_hi = share ? ((wave + 1) * gq < ngr ? (wave + 1) * gq : ngr) : ngr;
+  const int dt_lo = 4 * g_lo, dt_hi = 4 * g_hi < ct ? 4 * g_hi : ct;
   // with the rows shared out over nsplit blocks (blockIdx.z), each takes a run of whole steps
   const int nsteps = (kmax - kmin) / KSTEP + 1;
   const int per = (nsteps + nsplit - 1) / nsplit;
@@ -148,17 +151,21 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
     // a wavefront none of whose queries sees a row of this step waits for the next
     const bool step_on = wave_on && s0 <= pos0 + ti_hi && (window <= 0 || s0 + KSTEP - 1 > pos0 + ti_lo - window);
     if (!step_on) continue;
+    // (products that follow each other in the code belong to different accumulators: one that waits for the result of
+    // the one before it would leave the matrix cores idle for its whole latency)
     f32x4_t st[NB];
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      st[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int b = 0; b < NB; ++b) st[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kk = 0; kk < DK; ++kk)
-        if (32 * kk < D) {
-          const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks + (size_t)(16 * b + r16) * krow + 32 * kk + 8 * g);
-          st[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[kk], st[b], 0, 0, 0);
-        }
-    }
+    for (int kk = 0; kk < DK; ++kk)
+      if (32 * kk < D) {
+        bf16x8_t a[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+          a[b] = *reinterpret_cast<const bf16x8_t*>(ks + (size_t)(16 * b + r16) * krow + 32 * kk + 8 * g);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) st[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[b], qf[kk], st[b], 0, 0, 0);
+      }
     float mstep = -INFINITY;
 #pragma unroll
     for (int b = 0; b < NB; ++b)
@@ -189,22 +196,32 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
     psum = group4_sum(psum);
     lrun = lrun * alpha + psum;
     mrun = mnew;
+    // value columns in groups of four tiles: eight independent products side by side (four tiles, each with the
+    // weights' first and second term)
 #pragma unroll
-    for (int dt = 0; dt < CT; ++dt)
-      if (dt >= dt_lo && dt < dt_hi) {
-        f32x4_t a4 = acc[dt];
+    for (int g4 = 0; g4 < CT / 4; ++g4)
+      if (g4 >= g_lo && g4 < g_hi) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) a4[e] *= alpha;
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[4 * g4 + u][e] *= alpha;
 #pragma unroll
         for (int ch = 0; ch < NC; ++ch) {
-          const uint16_t* vr = vt + (size_t)(16 * dt + r16) * VROW + 32 * ch + 4 * g;
-          const u32x2_t v0 = *reinterpret_cast<const u32x2_t*>(vr);
-          const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(vr + 16);
-          const bf16x8_t a = __builtin_bit_cast(bf16x8_t, (u32x4_t{v0.x, v0.y, v1.x, v1.y}));
-          a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, phi[ch], a4, 0, 0, 0);
-          a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, plo[ch], a4, 0, 0, 0);
+          bf16x8_t a[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const uint16_t* vr = vt + (size_t)(16 * (4 * g4 + u) + r16) * VROW + 32 * ch + 4 * g;
+            const u32x2_t v0 = *reinterpret_cast<const u32x2_t*>(vr);
+            const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(vr + 16);
+            a[u] = __builtin_bit_cast(bf16x8_t, (u32x4_t{v0.x, v0.y, v1.x, v1.y}));
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            acc[4 * g4 + u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], phi[ch], acc[4 * g4 + u], 0, 0, 0);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            acc[4 * g4 + u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], plo[ch], acc[4 * g4 + u], 0, 0, 0);
         }
-        acc[dt] = a4;
       }
   }
   if (!valid) return;
@@ -288,12 +305,12 @@ extern "C" int gs_attention_latent_mfma(const void* qa, const void* cache, const
   GS_REQUIRE(hgroups <= 65535, "attention_latent_mfma: too many heads");
   dim3 grid(ntiles, hgroups, nsplit);
   if (c <= 128 && D <= 32 * (8 / 2 + 2)) {
-    const size_t lds = (size_t)64 * (Dp + 8) * 2 + (size_t)c * (64 + 4) * 2;
+    const size_t lds = (size_t)64 * (Dp + 8) * 2 + (size_t)((c + 63) & ~63) * (64 + 4) * 2;
     attention_latent_mfma_kernel<8, 64><<<grid, 256, lds, stream>>>(
         (const bf16*)qa, (const bf16*)cache, positions, tile_seq, tile_row, tile_n, block_table, max_blocks, page_size,
         window, scale, (bf16*)out, part_o, part_ml, nsplit, rows_total, H, HB, c, D);
   } else {
-    const size_t lds = (size_t)32 * (Dp + 8) * 2 + (size_t)c * (32 + 4) * 2;
+    const size_t lds = (size_t)32 * (Dp + 8) * 2 + (size_t)((c + 63) & ~63) * (32 + 4) * 2;
     static bool raised = false;
     if (!raised) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_latent_mfma_kernel<32, 32>),
