@@ -253,22 +253,24 @@ __global__ __launch_bounds__(256) void attention_latent_mfma_kernel(
 // that walked a row's keys in parts, added in the order of the parts.
 __global__ void attention_latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                               int nsplit, int rows_total, int c, bf16* __restrict__ out) {
-  const int row = blockIdx.x;
-  float M = -INFINITY;
-  for (int z = 0; z < nsplit; ++z) M = fmaxf(M, part_ml[((size_t)z * rows_total + row) * 2]);
-  float L = 0.f;
-  for (int z = 0; z < nsplit; ++z) {
-    const float* ml = part_ml + ((size_t)z * rows_total + row) * 2;
-    L += ml[1] * __builtin_amdgcn_exp2f(ml[0] - M);
+  __shared__ float wz[64];           // the parts' weights 2^(m_z - M) / L (at most 64 parts)
+  const int row = blockIdx.x, lane = threadIdx.x & 63;
+  // every wavefront of the block finds the weights itself: lane z holds part z
+  float m = -INFINITY, l = 0.f;
+  if (lane < nsplit) {
+    const float* ml = part_ml + ((size_t)lane * rows_total + row) * 2;
+    m = ml[0];
+    l = ml[1];
   }
-  const float inv = 1.0f / L;
+  const float M = wave_max(m);
+  const float w = lane < nsplit ? __builtin_amdgcn_exp2f(m - M) : 0.f;
+  const float L = wave_sum(l * w);
+  if (threadIdx.x < 64) wz[lane] = w / L;
+  __syncthreads();
   for (int j = threadIdx.x; j < c; j += blockDim.x) {
     float a = 0.f;
-    for (int z = 0; z < nsplit; ++z) {
-      const size_t prow = (size_t)z * rows_total + row;
-      a += part_o[prow * c + j] * __builtin_amdgcn_exp2f(part_ml[prow * 2] - M);
-    }
-    out[(size_t)row * c + j] = f32_to_bf16(a * inv);
+    for (int z = 0; z < nsplit; ++z) a += part_o[((size_t)z * rows_total + row) * c + j] * wz[z];
+    out[(size_t)row * c + j] = f32_to_bf16(a);
   }
 }
 

@@ -420,3 +420,22 @@ def test_greedy_generation_through_the_session(name, folders):
             assert all(supported(lg[i - 1], g[i], 0.5) for i in range(len(p), len(g)))
     finally:
         session.close()
+
+
+def test_the_command_line_serves_a_makuzen_folder(folders):
+    """``python -m gesso_amd --model DIR`` picks the model class by the folder's config.json; float32 gives the plain
+    model's tokens, also for a sampled request's first tokens being among the plain model's likely ones."""
+    import json
+    import os
+    import subprocess
+    import sys
+    cfg, _ = CONFIGS["D"]
+    model_dir = write_tiny(folders, "D", torch.float32)
+    prompt = random_ids(19, cfg.vocab, 77)
+    want = P.greedy(P.read_config(model_dir), P.read_weights(model_dir), prompt, 24)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-m", "gesso_amd", "--model", model_dir, "--dtype", "float32", "--prompt-ids",
+                        ",".join(str(t) for t in prompt), "--max-new-tokens", "24", "--n-ctx", "128"],
+                       capture_output=True, text=True, cwd=root, timeout=240, env=dict(os.environ, PYTHONPATH=root))
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert json.loads(r.stdout.strip().splitlines()[-1])["ids"] == [want]
