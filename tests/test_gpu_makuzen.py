@@ -463,3 +463,61 @@ def test_seventy_requests_at_once_decode_through_the_loop_for_many_rows(folders)
         assert all(supported(lg[j - 1], got[i][j], 0.5) for j in range(len(prompts[i]), len(got[i]))), i
     lg = P.forward(pc, pw, alone).numpy()
     assert all(supported(lg[j - 1], alone[j], 0.5) for j in range(len(prompts[0]), len(alone)))
+
+
+def random_makuzen(seed: int):
+    """A configuration drawn from a seed: two to four layers that differ from one another, sizes with and without
+    whole tiles, windows shorter and longer than the sequences or none, one to all experts used, layers without a
+    feed-forward or without a shared expert, rotation with and without slowed pairs."""
+    import random
+    from gesso_amd.config import LatentAttentionConfig, MakuzenConfig, MakuzenLayer, TableMoEConfig, YarnScaling
+    rng = random.Random(seed)
+    width = rng.choice([64, 72, 96, 128, 160, 256])
+    layers = []
+    for _ in range(rng.randint(2, 4)):
+        rot = rng.choice([2, 4, 8, 16, 32])
+        experts = rng.randint(1, 12)
+        mixer = LatentAttentionConfig(
+            heads=rng.choice([1, 2, 3, 4, 6, 8]), dim=rng.choice([8, 12, 16, 24, 32, 64]), rot_dim=rot,
+            vdim=rng.choice([8, 16, 20, 32, 64]), q_rank=rng.choice([16, 24, 40, 64, 96]),
+            kv_rank=rng.choice([16, 32, 36, 48, 64, 80, 128]), scale=rng.choice([0.08, 0.15, 0.25]),
+            rot_base=rng.choice([1e3, 1e4, 5e5]),
+            scaling=None if rng.random() < 0.4 else YarnScaling(rng.choice([2.0, 4.0, 8.0]), rng.choice([16.0, 64.0, 256.0]),
+                                                                rng.choice([4.0, 8.0, 32.0]), rng.choice([1.0, 2.0])),
+            window=rng.choice([None, 3, 16, 33, 64, 72, 150]))
+        mlp = None if rng.random() < 0.2 else TableMoEConfig(experts=experts, top=rng.randint(1, min(3, experts)),
+                                                             ff=rng.choice([8, 24, 32, 64]),
+                                                             shared_ff=rng.choice([None, 16, 40, 128]))
+        layers.append(MakuzenLayer(mixer, mlp))
+    return MakuzenConfig(vocab=rng.choice([97, 200, 333, 512]), width=width, layers=tuple(layers),
+                         embedding_scale=rng.choice([0.5, 1.0, 3.0]), norm_eps=rng.choice([1e-5, 1e-6, 1e-4]),
+                         residual_mult=rng.choice([0.25, 0.5, 1.0]), max_position=512)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", [31, 32, 33, 34, 35, 36])
+def test_replay_of_configurations_drawn_at_random(seed, dtype, tmp_path):
+    import random
+    from gesso_amd.weights import write_model_folder
+    cfg = random_makuzen(seed)
+    rng = random.Random(seed)
+    model_dir = write_model_folder(str(tmp_path / "m"), cfg, seed, torch.float32 if dtype == "float32" else torch.bfloat16,
+                                   std=STD)
+    lens = [rng.randint(1, 4), rng.randint(20, 60), rng.randint(70, 120), rng.randint(130, 210)]
+    seqs = {f"s{i}": random_ids(n, cfg.vocab, seed * 10 + i) for i, n in enumerate(lens)}
+    plain = R.Plain(model_dir, seqs, dtype)
+    ways = {"whole": R.trace_whole, "tail": lambda s: R.trace_tail(s, tail=40), "portions": R.trace_portions,
+            "mixed": lambda s: R.trace_mixed(s, seed=seed)}
+    big = R.Trace()
+    for way, make in ways.items():
+        t = make({f"{way}.{k}": v for k, v in seqs.items()})
+        for rec, rows in zip(t.steps, t.rows):
+            big.steps.append(dict(rec, step=len(big.steps)))
+            big.rows.append(rows)
+        big.max_tokens = max(big.max_tokens, t.max_tokens)
+    got, rc = R.run_trace(model_dir, dtype, str(tmp_path / "out"), big, cfg.vocab, extra=["--poison"])
+    assert rc == 0
+    for way in ways:
+        mine = {k.split(".", 1)[1]: v for k, v in got.items() if k.startswith(way + ".")}
+        assert {k: len(v) for k, v in mine.items()} == {k: len(v) for k, v in seqs.items()}, way
+        plain.check(mine, f"seed {seed} {way}")
