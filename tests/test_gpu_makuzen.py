@@ -242,7 +242,7 @@ class Tokens:
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("E,top,F,shared,H", [(5, 2, 40, 56, 96), (3, 1, 24, None, 96), (4, 4, 8, 8, 64), (7, 3, 20, 36, 100),
-                                              (6, 2, 64, 128, 256)])
+                                              (6, 2, 96, 160, 384)])
 def test_table_routed_experts_alone(dtype, E, top, F, shared, H):
     from gesso_amd.config import TableMoESpec
     from test_gpu_parts import Harness
