@@ -311,6 +311,20 @@ extern "C" int gs_attention_latent_mfma(const void* qa, const void* cache, const
     attention_latent_mfma_kernel<8, 64><<<grid, 256, lds, stream>>>(
         (const bf16*)qa, (const bf16*)cache, positions, tile_seq, tile_row, tile_n, block_table, max_blocks, page_size,
         window, scale, (bf16*)out, part_o, part_ml, nsplit, rows_total, H, HB, c, D);
+  } else if (c <= 256 && D <= 32 * (16 / 2 + 2)) {
+    // latents up to 256: half the accumulators of the widest form, so steps of 64 rows fit
+    const size_t lds = (size_t)64 * (Dp + 8) * 2 + (size_t)((c + 63) & ~63) * (64 + 4) * 2;
+    static bool raised_mid = false;
+    if (!raised_mid) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_latent_mfma_kernel<16, 64>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+      GS_REQUIRE(e == hipSuccess, "attention_latent_mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
+      raised_mid = true;
+    }
+    GS_REQUIRE(lds <= 96 * 1024, "attention_latent_mfma: %zu bytes of LDS", lds);
+    attention_latent_mfma_kernel<16, 64><<<grid, 256, lds, stream>>>(
+        (const bf16*)qa, (const bf16*)cache, positions, tile_seq, tile_row, tile_n, block_table, max_blocks, page_size,
+        window, scale, (bf16*)out, part_o, part_ml, nsplit, rows_total, H, HB, c, D);
   } else {
     const size_t lds = (size_t)32 * (Dp + 8) * 2 + (size_t)((c + 63) & ~63) * (32 + 4) * 2;
     static bool raised = false;
