@@ -28,16 +28,19 @@ from .pages import PagePool, SlotPool
 RELEASED = -1   # a block-table entry whose page the window has passed
 
 
+# A cache is named by the position in the schedule of the call that keeps it, or by ``(position, k)`` for the k-th
+# cache of a call that keeps several (a mixer made of two mixers).
+
 @dataclass(frozen=True)
 class PagedGroup:
     index: int
     need: PagedKV
-    members: Tuple[int, ...]        # positions in the schedule that keep their cache here
+    members: Tuple[Hashable, ...]   # the caches that lie here
 
 
 @dataclass(frozen=True)
 class SlotMember:
-    call: int                        # position in the schedule
+    call: Hashable                   # the cache's name
     need: SlotState
 
 
@@ -47,21 +50,32 @@ class CacheLayout:
 
     paged: Tuple[PagedGroup, ...]
     slots: Tuple[SlotMember, ...]
-    group_of_call: Dict[int, int]    # schedule position -> paged group index (own caches only)
+    group_of_call: Dict[Hashable, int]   # cache name -> paged group index (own caches only)
     source_of_call: Dict[int, int]   # schedule position -> the position whose cache it uses
+    parts_of_call: Dict[int, int] = field(default_factory=dict)   # schedule position -> how many caches it keeps, where several
 
     @staticmethod
     def plan(needs: Sequence[Optional[object]], cache_of: Sequence[Optional[int]]) -> "CacheLayout":
-        """``needs[i]``: what call ``i`` keeps (None if nothing or if it reads ``cache_of[i]``)."""
-        groups: Dict[PagedKV, List[int]] = {}
+        """``needs[i]``: what call ``i`` keeps (None if nothing or if it reads ``cache_of[i]``); a tuple: several caches."""
+        groups: Dict[PagedKV, List[Hashable]] = {}
         slots: List[SlotMember] = []
-        for i, need in enumerate(needs):
+        several: Dict[int, int] = {}
+
+        def place(name, need, i):
             if isinstance(need, PagedKV):
-                groups.setdefault(need, []).append(i)
+                groups.setdefault(need, []).append(name)
             elif isinstance(need, SlotState):
-                slots.append(SlotMember(i, need))
+                slots.append(SlotMember(name, need))
             elif need is not None:
                 raise InvalidPlan(f"schedule entry {i} asks for an unknown kind of cache: {need!r}")
+
+        for i, need in enumerate(needs):
+            if isinstance(need, (tuple, list)):
+                several[i] = len(need)
+                for k, sub in enumerate(need):
+                    place((i, k), sub, i)
+            else:
+                place(i, need, i)
         paged = tuple(PagedGroup(g, need, tuple(m)) for g, (need, m) in enumerate(groups.items()))
         group_of = {c: g.index for g in paged for c in g.members}
         source = {}
@@ -70,7 +84,7 @@ class CacheLayout:
             while cache_of[s] is not None:
                 s = cache_of[s]
             source[i] = s
-        return CacheLayout(paged, tuple(slots), group_of, source)
+        return CacheLayout(paged, tuple(slots), group_of, source, several)
 
 
 @dataclass
@@ -184,10 +198,9 @@ class CacheManager:
         if -(-rc.length // self.page_size) > min((len(t) for t in rc.tables), default=1 << 60):
             raise InvalidPlan(f"request {rid!r} advanced beyond its reserved pages")
         for g, group in enumerate(self.layout.paged):
-            w = group.need.window
-            if w is None:
+            if group.need.window is None and group.need.chunk is None:
                 continue
-            first_needed = rc.length - w + 1          # oldest key the next query reads
+            first_needed = group.need.first_needed(rc.length)     # oldest key the next query reads
             passed = max(0, first_needed) // self.page_size
             table = rc.tables[g]
             gone = [table[b] for b in range(min(passed, len(table))) if table[b] != RELEASED]

@@ -85,6 +85,12 @@ class CacheStorage:
         """The cache of schedule position ``call`` (its own, or the one it reads)."""
         src = self.layout.source_of_call[call]
         write = src == call
+        several = self.layout.parts_of_call.get(src)
+        if several is not None:
+            return tuple(self._view((src, k), write, block_tables) for k in range(several))
+        return self._view(src, write, block_tables)
+
+    def _view(self, src, write: bool, block_tables) -> Optional[object]:
         if src in self.layout.group_of_call:
             g = self.layout.group_of_call[src]
             i = self.member_index[src]

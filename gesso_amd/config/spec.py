@@ -21,9 +21,13 @@ from typing import Any, Mapping, Optional, Tuple
 
 @dataclass(frozen=True)
 class RMSNormSpec:
+    """``x / sqrt(mean(x^2) + eps) * (offset + w)``: ``offset`` is what the stored weight lies around (0: the weight
+    itself multiplies; 1: a weight stored around zero)."""
+
     size: int
     eps: float
     kind: str = "rmsnorm"
+    offset: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -64,6 +68,27 @@ class ScaledRopeSpec:
 
 
 @dataclass(frozen=True)
+class StretchedRopeSpec:
+    """Rotary encoding whose frequencies are stretched by wavelength for contexts longer than ``original``.
+
+    Pair ``i`` turns by ``f_i = theta^(-2i/rotary_dim)`` a position; with the wavelength ``l_i = 2 pi / f_i`` the pair
+    keeps ``f_i`` where ``l_i < original / high``, gets ``f_i / factor`` where ``l_i > original / low``, and between the
+    two, with ``s = (original / l_i - low) / (high - low)``, the blend ``(1 - s) f_i / factor + s f_i``.
+    ``factor = None``: plain rotation."""
+
+    head_dim: int
+    rotary_dim: int
+    theta: float
+    max_position: int
+    factor: Optional[float] = None
+    original: float = 0.0
+    low: float = 1.0
+    high: float = 4.0
+    layout: str = "half"
+    kind: str = "stretched_rope"
+
+
+@dataclass(frozen=True)
 class NoPositionSpec:
     kind: str = "none"
 
@@ -80,6 +105,11 @@ class AttentionSpec:
     bias: bool = False
     scale: Optional[float] = None      # None = 1/sqrt(head_dim)
     kind: str = "attention"
+    value_dim: Optional[int] = None    # width of a value head; None = head_dim
+    chunk: Optional[int] = None        # positions are cut into runs of this many from 0 on, a query sees its own run
+    sink: bool = False                 # the softmax's denominator has one more term, exp(0), which has no value
+    value_position: Any = None         # a position-encoding spec: values are cached turned by their own position, a
+                                       # head's weighted sum is turned back by the query's
 
 
 @dataclass(frozen=True)
@@ -106,6 +136,44 @@ class LatentAttentionSpec:
 
 
 @dataclass(frozen=True)
+class LinearAttentionSpec:
+    """Attention without a softmax, through a matrix state per head that fades by a fixed factor a token:
+    ``S_t = decay_h S_(t-1) + k_t v_t^T`` (``key_dim x value_dim``, float32, zero at a request's start),
+    ``o_t = S_t^T q_t``.
+
+    ``activation``: applied to the q, k and v products (``"silu"`` or None).  ``position``: turns q and k (a
+    position-encoding spec).  ``key_scale``: multiplies k after the turn.  ``out_norm``: ``"joint"`` = the heads' outputs
+    side by side are normed as one row with a weight, ``"head"`` = each head's output is divided by its own root mean
+    square, no weight.  ``gate``: the normed row is multiplied by this function of a further product of the input
+    (``"sigmoid"`` or ``"silu"``)."""
+
+    hidden: int
+    n_heads: int
+    key_dim: int
+    value_dim: int
+    decay: Tuple[float, ...]
+    eps: float
+    position: Any = NoPositionSpec()
+    activation: Optional[str] = None
+    key_scale: float = 1.0
+    out_norm: str = "joint"
+    gate: str = "sigmoid"
+    kind: str = "linear_attention"
+
+
+@dataclass(frozen=True)
+class MixerPairSpec:
+    """Two mixers side by side that read the same input: ``left_scale * left(x) + right_scale * right(x)``.  Each keeps
+    its own cache."""
+
+    left: Any
+    right: Any
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    kind: str = "mixer_pair"
+
+
+@dataclass(frozen=True)
 class ShortConvSpec:
     hidden: int
     width: int                         # taps, the current input included (conv_L_cache)
@@ -118,6 +186,18 @@ class SwiGLUSpec:
     hidden: int
     intermediate: int
     kind: str = "swiglu"
+
+
+@dataclass(frozen=True)
+class GatedMLPSpec:
+    """``W_down (act(W_gate x + b_gate) * (W_up x + b_up)) + b_down``; ``activation``: ``"gelu_tanh"``
+    (``0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))``) or ``"silu"``; ``bias``: whether the three products have one."""
+
+    hidden: int
+    intermediate: int
+    activation: str = "gelu_tanh"
+    bias: bool = True
+    kind: str = "gated_mlp"
 
 
 @dataclass(frozen=True)
@@ -169,6 +249,19 @@ class OutNormBlockSpec:
 
 
 @dataclass(frozen=True)
+class ParallelBlockSpec:
+    """One block whose sub-layers read the same stream: ``h += mixer(norm_a(h)) + ffn(norm_b(h))``.  ``names`` as in
+    :class:`BlockSpec`."""
+
+    mixer: Any
+    mixer_norm: Any
+    ffn: Any                           # None = no feed-forward in this block
+    ffn_norm: Any
+    names: Mapping[str, str] = field(compare=False, hash=False, default_factory=dict)
+    kind: str = "parallel"
+
+
+@dataclass(frozen=True)
 class LayerCall:
     """One entry of the run order: block ``layer`` runs here.
 
@@ -195,6 +288,8 @@ class ModelSpec:
     eos_token_ids: Tuple[int, ...] = ()
     ignored_tensors: Tuple[str, ...] = ()   # suffixes that a file may hold and nobody reads
     embed_scale: Optional[float] = None     # the embedding rows are multiplied by this (None: as they are)
+    embed_norm: Any = None                  # a norm spec: the embedding rows are normed before the first block
+                                            # (its tensors under names "embed_norm.<local>")
     logit_softcap: Optional[float] = None   # logits = cap * tanh(logits / cap) (None: as they are)
 
     def __post_init__(self):

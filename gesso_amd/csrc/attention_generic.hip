@@ -10,8 +10,14 @@
 //
 //   s_u = (q . k_u) * scale;  p_u = exp(s_u - max);  o = sum_u p_u v_u / sum_u p_u
 //
-// q (T, q_stride) with head h at columns [h d, (h+1) d); out (T, nh d); caches
-// (num_pages, nkv, page_size, d).
+// q (T, q_stride) with head h at columns [h d, (h+1) d); out (T, nh vd); key cache
+// (num_pages, nkv, page_size, d), value cache (num_pages, nkv, page_size, vd).
+//
+// Further rules, each off unless asked for.  chunk > 0: positions are cut into runs of `chunk` from 0 on and a query
+// sees only its own run, lo = max(lo, p - p % chunk).  sink: the denominator has one more term, exp(0 - max), which
+// has no value: o = sum_u p_u v_u / (exp(-max) + sum_u p_u), the maximum taken over the scores and 0.  Value tables
+// (max_position, vd/2): the cached values were turned by their own positions (rope_kv.hip), and the head's sum is
+// turned back by the query's position, pair (a, b) -> (a cos + b sin, b cos - a sin), before it is stored.
 #include "common.h"
 
 #define GS_ATTN_MAX_D 256
@@ -21,7 +27,9 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, int q_stride, 
                                          const T* __restrict__ vcache, const int* __restrict__ positions,
                                          const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                                          int max_blocks, int page_size, int window, float scale, T* __restrict__ out,
-                                         int nh, int nkv, int d) {
+                                         int nh, int nkv, int d, int vd, int chunk, int sink,
+                                         const float* __restrict__ vcos, const float* __restrict__ vsin,
+                                         int interleaved) {
   __shared__ float qs[GS_ATTN_MAX_D];
   __shared__ float ps[64];
   __shared__ long rowoff[64];
@@ -35,7 +43,9 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, int q_stride, 
   __syncthreads();
 
   int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
-  float m = -INFINITY, l = 0.f;
+  if (chunk > 0 && pos - pos % chunk > lo) lo = pos - pos % chunk;
+  // with a sink the running maximum starts at the sink's score and the sum at its term
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
   float acc[GS_ATTN_MAX_D / 64];
 #pragma unroll
   for (int i = 0; i < GS_ATTN_MAX_D / 64; ++i) acc[i] = 0.f;
@@ -46,8 +56,8 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, int q_stride, 
     long off = 0;
     if (u <= pos) {
       int page = bt[u / page_size];
-      off = (((long)page * nkv + kvh) * page_size + u % page_size) * d;
-      const T* kr = kcache + off;
+      off = ((long)page * nkv + kvh) * page_size + u % page_size;
+      const T* kr = kcache + off * d;
       float dot = 0.f;
       for (int j = 0; j < d; ++j) dot += qs[j] * to_f32(kr[j]);
       s = dot * scale;
@@ -65,25 +75,48 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, int q_stride, 
 #pragma unroll
     for (int i = 0; i < GS_ATTN_MAX_D / 64; ++i) {
       int j = lane + 64 * i;
-      if (j < d) {
+      if (j < vd) {
         float a = acc[i] * alpha;
-        for (int k = 0; k < nk; ++k) a += ps[k] * to_f32(vcache[rowoff[k] + j]);
+        for (int k = 0; k < nk; ++k) a += ps[k] * to_f32(vcache[rowoff[k] * vd + j]);
         acc[i] = a;
       }
     }
   }
   float inv = 1.0f / l;
+  if (vcos) {
+    // the sum of turned values is turned back by the query's position
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < GS_ATTN_MAX_D / 64; ++i) {
+      int j = lane + 64 * i;
+      if (j < vd) qs[j] = acc[i] * inv;
+    }
+    __syncthreads();
+    const int vh = vd >> 1;
+    for (int i = lane; i < vh; i += 64) {
+      const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + vh;
+      const float a = qs[ia], b = qs[ib];
+      const float c = vcos[(size_t)pos * vh + i], sn = vsin[(size_t)pos * vh + i];
+      out[((size_t)t * nh + h) * vd + ia] = from_f32<T>(a * c + b * sn);
+      out[((size_t)t * nh + h) * vd + ib] = from_f32<T>(b * c - a * sn);
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < GS_ATTN_MAX_D / 64; ++i) {
     int j = lane + 64 * i;
-    if (j < d) out[((size_t)t * nh + h) * d + j] = from_f32<T>(acc[i] * inv);
+    if (j < vd) out[((size_t)t * nh + h) * vd + j] = from_f32<T>(acc[i] * inv);
   }
 }
 
 extern "C" int gs_attention_generic(const void* q, int q_stride, const void* kcache, const void* vcache, int dtype,
                                     const int* positions, const int* seq_of_token, const int* block_table,
                                     int max_blocks, int page_size, int window, float scale, void* out, int ntok,
-                                    int nh, int nkv, int d, hipStream_t stream) {
+                                    int nh, int nkv, int d, int vd, int chunk, int sink, const float* vcos,
+                                    const float* vsin, int interleaved, hipStream_t stream) {
+  GS_REQUIRE(vd > 0 && vd <= GS_ATTN_MAX_D, "attention: value width %d outside 1..%d", vd, GS_ATTN_MAX_D);
+  GS_REQUIRE(chunk >= 0, "attention: bad chunk %d", chunk);
+  GS_REQUIRE((vcos == nullptr) == (vsin == nullptr) && (!vcos || vd % 2 == 0), "attention: value tables come together, for even widths");
   GS_REQUIRE(ntok >= 0 && nh > 0 && nkv > 0 && d > 0, "attention: bad sizes T=%d nh=%d nkv=%d d=%d", ntok, nh, nkv, d);
   GS_REQUIRE(nh % nkv == 0, "attention: %d query heads are no multiple of %d key heads", nh, nkv);
   GS_REQUIRE(d <= GS_ATTN_MAX_D, "attention: head width %d above the kernel's limit %d", d, GS_ATTN_MAX_D);
@@ -96,12 +129,14 @@ extern "C" int gs_attention_generic(const void* q, int q_stride, const void* kca
     attention_generic_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, q_stride, (const float*)kcache,
                                                               (const float*)vcache, positions, seq_of_token,
                                                               block_table, max_blocks, page_size, window, scale,
-                                                              (float*)out, nh, nkv, d);
+                                                              (float*)out, nh, nkv, d, vd, chunk, sink, vcos, vsin,
+                                                              interleaved);
   else if (dtype == GS_BF16)
     attention_generic_kernel<bf16><<<grid, 64, 0, stream>>>((const bf16*)q, q_stride, (const bf16*)kcache,
                                                              (const bf16*)vcache, positions, seq_of_token,
                                                              block_table, max_blocks, page_size, window, scale,
-                                                             (bf16*)out, nh, nkv, d);
+                                                             (bf16*)out, nh, nkv, d, vd, chunk, sink, vcos, vsin,
+                                                             interleaved);
   else
     GS_REQUIRE(false, "attention: unknown dtype %d", dtype);
   GS_LAUNCH_CHECK("attention_generic");

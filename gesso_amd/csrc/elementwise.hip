@@ -19,7 +19,7 @@ void gs_set_error(const char* fmt, ...) {
 
 extern "C" const char* gs_last_error() { return g_err; }
 
-extern "C" int gs_abi_version() { return 10; }
+extern "C" int gs_abi_version() { return 11; }
 
 // ------------------------------------------------------------------ embedding
 
@@ -606,5 +606,141 @@ extern "C" int gs_fill_rows(void* pool, int dtype, const int* ids, int n, long r
   else
     GS_REQUIRE(false, "fill_rows: unknown dtype %d", dtype);
   GS_LAUNCH_CHECK("fill_rows");
+  return 0;
+}
+
+// ------------------------------------------------------------------ two adds + two RMSNorms of one row
+
+// One block per row: x = res (+ d1) (+ d2), written back; out1 = x * inv_rms(x) * w1, out2 = x * inv_rms(x) * w2
+// (out2 and w2 may be absent).  The block of a layer whose mixer and feed-forward both read the same stream, each
+// through a norm of its own, needs the stream's row once for both; the two results of the layer before are added on
+// the way.  The row stays in registers or LDS between the passes: rows up to 8192 values, else it is read again.
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_pair_kernel(float* __restrict__ res, const TD* __restrict__ d1, const TD* __restrict__ d2,
+                                        const float* __restrict__ w1, const float* __restrict__ w2, float eps,
+                                        TO* __restrict__ out1, TO* __restrict__ out2, int H) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  float* x = res + (size_t)r * H;
+  const TD* a = d1 ? d1 + (size_t)r * H : nullptr;
+  const TD* b = d2 ? d2 + (size_t)r * H : nullptr;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) {
+    float v = x[j];
+    if (a) v += to_f32(a[j]);
+    if (b) v += to_f32(b[j]);
+    if (a || b) x[j] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = norm_inverse(ss, (float)H, eps);
+  TO* o1 = out1 + (size_t)r * H;
+  TO* o2 = out2 ? out2 + (size_t)r * H : nullptr;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) {
+    const float v = x[j] * inv;                 // (this thread wrote x[j] itself)
+    o1[j] = from_f32<TO>(v * w1[j]);
+    if (o2) o2[j] = from_f32<TO>(v * w2[j]);
+  }
+}
+
+extern "C" int gs_add_rmsnorm_pair(float* res, const void* d1, const void* d2, int delta_dtype, const float* w1,
+                                   const float* w2, float eps, void* out1, void* out2, int out_dtype, int T, int H,
+                                   hipStream_t stream) {
+  GS_REQUIRE(T >= 0 && H > 0, "add_rmsnorm_pair: bad sizes rows=%d H=%d", T, H);
+  GS_REQUIRE(eps > 0.f, "add_rmsnorm_pair: eps must be positive");
+  GS_REQUIRE(w1 && out1 && ((w2 == nullptr) == (out2 == nullptr)), "add_rmsnorm_pair: a weight for every output");
+  if (T == 0) return 0;
+  const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
+#define GS_RUN(TD, TO)                                                                                             \
+  add_rmsnorm_pair_kernel<TD, TO><<<T, threads, 0, stream>>>(res, (const TD*)d1, (const TD*)d2, w1, w2, eps,       \
+                                                              (TO*)out1, (TO*)out2, H)
+  if (delta_dtype == GS_F32 && out_dtype == GS_F32)
+    GS_RUN(float, float);
+  else if (delta_dtype == GS_BF16 && out_dtype == GS_BF16)
+    GS_RUN(bf16, bf16);
+  else if (delta_dtype == GS_F32 && out_dtype == GS_BF16)
+    GS_RUN(float, bf16);
+  else if (delta_dtype == GS_BF16 && out_dtype == GS_F32)
+    GS_RUN(bf16, float);
+  else
+    GS_REQUIRE(false, "add_rmsnorm_pair: unknown dtypes %d %d", delta_dtype, out_dtype);
+#undef GS_RUN
+  GS_LAUNCH_CHECK("add_rmsnorm_pair");
+  return 0;
+}
+
+// ------------------------------------------------------------------ gated activation with biases
+
+// in (T, 2F) = gate | up (a product's float32 sums or rounded rows), bias (2F) float32 or absent:
+//   out[t, j] = act(gate[t, j] + bias[j]) * (up[t, j] + bias[F + j])
+// act 0: silu, z / (1 + exp(-z)); act 1: the tanh form of gelu, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+__device__ __forceinline__ float gated_act(float z, int act) {
+  if (act == 0) return z / (1.0f + expf(-z));
+  const float u = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+  return 0.5f * z * (1.0f + tanhf(u));
+}
+
+template <typename TI, typename TO>
+__global__ void gated_act_kernel(const TI* __restrict__ in, const float* __restrict__ bias, TO* __restrict__ out, int F,
+                                 long n, int act) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const long t = i / F;
+  const int j = (int)(i - t * F);
+  float g = to_f32(in[t * 2 * F + j]), u = to_f32(in[t * 2 * F + F + j]);
+  if (bias) {
+    g += bias[j];
+    u += bias[F + j];
+  }
+  out[i] = from_f32<TO>(gated_act(g, act) * u);
+}
+
+extern "C" int gs_gated_act(const void* in, int in_dtype, const float* bias, void* out, int out_dtype, int T, int F,
+                            int act, hipStream_t stream) {
+  GS_REQUIRE(T >= 0 && F > 0, "gated_act: bad sizes T=%d F=%d", T, F);
+  GS_REQUIRE(act == 0 || act == 1, "gated_act: unknown activation %d", act);
+  const long n = (long)T * F;
+  if (n == 0) return 0;
+  const int blocks = gs_ceil_div(n, 256);
+#define GS_RUN(TI, TO) gated_act_kernel<TI, TO><<<blocks, 256, 0, stream>>>((const TI*)in, bias, (TO*)out, F, n, act)
+  if (in_dtype == GS_F32 && out_dtype == GS_F32)
+    GS_RUN(float, float);
+  else if (in_dtype == GS_F32 && out_dtype == GS_BF16)
+    GS_RUN(float, bf16);
+  else if (in_dtype == GS_BF16 && out_dtype == GS_BF16)
+    GS_RUN(bf16, bf16);
+  else
+    GS_REQUIRE(false, "gated_act: unknown dtypes %d %d", in_dtype, out_dtype);
+#undef GS_RUN
+  GS_LAUNCH_CHECK("gated_act");
+  return 0;
+}
+
+// ------------------------------------------------------------------ weighted sum of two results
+
+// out = sa * a + sb * b, elementwise in float32, rounded once.
+template <typename TI, typename TO>
+__global__ void scaled_sum_kernel(const TI* __restrict__ a, float sa, const TI* __restrict__ b, float sb,
+                                  TO* __restrict__ out, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_f32<TO>(sa * to_f32(a[i]) + sb * to_f32(b[i]));
+}
+
+extern "C" int gs_scaled_sum(const void* a, float sa, const void* b, float sb, int in_dtype, void* out, int out_dtype,
+                             long n, hipStream_t stream) {
+  GS_REQUIRE(n >= 0, "scaled_sum: bad size");
+  if (n == 0) return 0;
+  const int blocks = gs_ceil_div(n, 256);
+#define GS_RUN(TI, TO) scaled_sum_kernel<TI, TO><<<blocks, 256, 0, stream>>>((const TI*)a, sa, (const TI*)b, sb, (TO*)out, n)
+  if (in_dtype == GS_F32 && out_dtype == GS_F32)
+    GS_RUN(float, float);
+  else if (in_dtype == GS_F32 && out_dtype == GS_BF16)
+    GS_RUN(float, bf16);
+  else if (in_dtype == GS_BF16 && out_dtype == GS_BF16)
+    GS_RUN(bf16, bf16);
+  else
+    GS_REQUIRE(false, "scaled_sum: unknown dtypes %d %d", in_dtype, out_dtype);
+#undef GS_RUN
+  GS_LAUNCH_CHECK("scaled_sum");
   return 0;
 }

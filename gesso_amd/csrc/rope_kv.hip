@@ -9,6 +9,9 @@
 //   q is written back in place; k (after norm and rotation) and v (as it is) go to the cache:
 //   page = block_table[seq, pos / page_size], row = pos % page_size,
 //   cache (num_pages, nkv, page_size, d).
+// A value head may be vd wide instead of d (the row is then (nh + nkv) d + nkv vd wide, the value cache
+// (num_pages, nkv, page_size, vd)), and with value tables (max_position, vd/2) the values are cached turned by
+// their own position over their whole width, in the same layout of pairs; whoever sums them turns the sum back.
 // One wave per (token, head).  All arithmetic float32.
 #include "common.h"
 
@@ -18,26 +21,40 @@ __global__ void qknorm_rope_kv_kernel(T* __restrict__ qkv, const float* __restri
                                       int rotary_dim, int interleaved, const int* __restrict__ positions,
                                       const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                                       int max_blocks, int page_size, T* __restrict__ kcache, T* __restrict__ vcache,
-                                      int ntok, int nh, int nkv, int d, int write_kv) {
+                                      int ntok, int nh, int nkv, int d, int write_kv, int vd,
+                                      const float* __restrict__ vcos, const float* __restrict__ vsin) {
   int lane = threadIdx.x & 63;
   int heads = nh + 2 * nkv;
   long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (unit >= (long)ntok * heads) return;
   int t = (int)(unit / heads);
   int hh = (int)(unit - (long)t * heads);
-  T* x = qkv + ((size_t)t * heads + hh) * d;
+  const size_t row_len = (size_t)(nh + nkv) * d + (size_t)nkv * vd;
+  const bool is_v = hh >= nh + nkv;
+  T* x = qkv + (size_t)t * row_len + (is_v ? (size_t)(nh + nkv) * d + (size_t)(hh - nh - nkv) * vd : (size_t)hh * d);
   int pos = positions[t];
 
   T* dst = nullptr;  // cache row for k and v heads
   if (hh >= nh) {
     if (!write_kv) return;
-    int kvh = hh < nh + nkv ? hh - nh : hh - nh - nkv;
+    int kvh = is_v ? hh - nh - nkv : hh - nh;
     int page = block_table[(size_t)seq_of_token[t] * max_blocks + pos / page_size];
-    T* base = hh < nh + nkv ? kcache : vcache;
-    dst = base + (((size_t)page * nkv + kvh) * page_size + pos % page_size) * d;
+    T* base = is_v ? vcache : kcache;
+    dst = base + (((size_t)page * nkv + kvh) * page_size + pos % page_size) * (is_v ? vd : d);
   }
-  if (hh >= nh + nkv) {  // v: copy
-    for (int j = lane; j < d; j += 64) dst[j] = x[j];
+  if (is_v) {  // v: copy, or turn by the position over the whole width
+    if (!vcos) {
+      for (int j = lane; j < vd; j += 64) dst[j] = x[j];
+      return;
+    }
+    const int vh = vd >> 1;
+    for (int i = lane; i < vh; i += 64) {
+      const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + vh;
+      const float a = to_f32(x[ia]), b = to_f32(x[ib]);
+      const float c = vcos[(size_t)pos * vh + i], s = vsin[(size_t)pos * vh + i];
+      dst[ia] = from_f32<T>(a * c - b * s);
+      dst[ib] = from_f32<T>(a * s + b * c);
+    }
     return;
   }
 
@@ -135,7 +152,11 @@ extern "C" int gs_qknorm_rope_kv(void* qkv, int dtype, const float* qw, const fl
                                  const float* cos_t, const float* sin_t, int rotary_dim, int interleaved,
                                  int max_position, const int* positions, const int* seq_of_token, const int* block_table,
                                  int max_blocks, int page_size, void* kcache, void* vcache, int ntok, int nh, int nkv,
-                                 int d, int write_kv, hipStream_t stream) {
+                                 int d, int write_kv, int vd, const float* vcos, const float* vsin,
+                                 hipStream_t stream) {
+  GS_REQUIRE(vd > 0, "qknorm_rope_kv: values of width %d", vd);
+  GS_REQUIRE((vcos == nullptr) == (vsin == nullptr), "qknorm_rope_kv: the value tables come together");
+  GS_REQUIRE(!vcos || (vd % 2 == 0 && max_position > 0), "qknorm_rope_kv: turned values are of even width");
   GS_REQUIRE(ntok >= 0 && nh > 0 && nkv > 0 && d > 0, "qknorm_rope_kv: bad sizes T=%d nh=%d nkv=%d d=%d", ntok, nh,
              nkv, d);
   GS_REQUIRE(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0,
@@ -146,7 +167,7 @@ extern "C" int gs_qknorm_rope_kv(void* qkv, int dtype, const float* qw, const fl
   GS_REQUIRE((qw == nullptr) == (kw == nullptr), "qknorm_rope_kv: q and k norm weights come together");
   if (ntok == 0) return 0;
   long units = (long)ntok * (nh + 2 * nkv);
-  const bool vec = !interleaved && rotary_dim == d && (d == 16 || d == 32 || d == 64 || d == 128) && (dtype == GS_F32 || dtype == GS_BF16) &&
+  const bool vec = !interleaved && vd == d && !vcos && rotary_dim == d && (d == 16 || d == 32 || d == 64 || d == 128) && (dtype == GS_F32 || dtype == GS_BF16) &&
                    ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)kcache & 15) == 0 && ((uintptr_t)vcache & 15) == 0 &&
                    ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0 && ((uintptr_t)qw & 15) == 0 &&
                    ((uintptr_t)kw & 15) == 0;
@@ -174,7 +195,7 @@ extern "C" int gs_qknorm_rope_kv(void* qkv, int dtype, const float* qw, const fl
 #define GS_RUN(T)                                                                                               \
   qknorm_rope_kv_kernel<T><<<blocks, 256, 0, stream>>>((T*)qkv, qw, kw, eps, cos_t, sin_t, rotary_dim, interleaved, positions, \
                                                        seq_of_token, block_table, max_blocks, page_size,        \
-                                                       (T*)kcache, (T*)vcache, ntok, nh, nkv, d, write_kv)
+                                                       (T*)kcache, (T*)vcache, ntok, nh, nkv, d, write_kv, vd, vcos, vsin)
   if (dtype == GS_F32)
     GS_RUN(float);
   else if (dtype == GS_BF16)

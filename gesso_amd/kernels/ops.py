@@ -304,14 +304,27 @@ def short_conv(bcx, taps, bias, state, seq_of_token, q_start, slots, nseq: int, 
 ROPE_LAYOUTS = ("half", "interleaved")
 
 
+def _value_tables(vcos, vsin, vd):
+    """Checks the tables by which values are turned (``(P, vd/2)`` float32, both or neither)."""
+    _need((vcos is None) == (vsin is None), "the value tables come together")
+    if vcos is not None:
+        _dev(vcos, vsin)
+        _need(vd % 2 == 0 and vcos.dtype == torch.float32 and vsin.dtype == torch.float32 and vcos.shape == vsin.shape
+              and vcos.dim() == 2 and vcos.shape[1] == vd // 2, "value tables must be float32 (P, value width / 2)")
+
+
 def qknorm_rope_kv(qkv, q_weight, k_weight, eps, cos, sin, rotary_dim, positions, seq_of_token, block_table,
-                   page_size, kcache, vcache, nh, nkv, d, write_kv=True, layout: str = "half") -> None:
+                   page_size, kcache, vcache, nh, nkv, d, write_kv=True, layout: str = "half", vd: int = None,
+                   vcos=None, vsin=None) -> None:
     """Head norm and rotation of q (in place) and k; k and v written into the pages.  ``layout``: which features
-    form a rotation pair, ``"half"`` (i, i + rotary_dim/2) or ``"interleaved"`` (2i, 2i + 1)."""
+    form a rotation pair, ``"half"`` (i, i + rotary_dim/2) or ``"interleaved"`` (2i, 2i + 1).  ``vd``: the width of
+    a value head where it is not ``d``; ``vcos``, ``vsin`` ``(P, vd/2)``: the values are cached turned by their
+    position over their whole width."""
     _need(layout in ROPE_LAYOUTS, f"qknorm_rope_kv: pairs are laid out 'half' or 'interleaved', not {layout!r}")
     _dev(qkv, q_weight, k_weight, cos, sin, positions, seq_of_token, block_table, kcache, vcache)
+    vd = d if vd is None else int(vd)
     T = qkv.shape[0]
-    _need(qkv.shape == (T, (nh + 2 * nkv) * d), "qknorm_rope_kv: qkv must be (T, (nh + 2 nkv) d)")
+    _need(qkv.shape == (T, (nh + nkv) * d + nkv * vd), "qknorm_rope_kv: qkv must be (T, (nh + nkv) d + nkv vd)")
     for w in (q_weight, k_weight):
         _need(w is None or (w.dtype == torch.float32 and w.shape == (d,)), "qknorm_rope_kv: head norm weight must be float32 (d,)")
     max_pos = 0
@@ -319,38 +332,155 @@ def qknorm_rope_kv(qkv, q_weight, k_weight, eps, cos, sin, rotary_dim, positions
         _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape
               and cos.dim() == 2 and cos.shape[1] == rotary_dim // 2, "qknorm_rope_kv: tables must be float32 (P, rotary_dim/2)")
         max_pos = cos.shape[0]
+    _value_tables(vcos, vsin, vd)
+    if vcos is not None:
+        max_pos = vcos.shape[0] if not max_pos else min(max_pos, vcos.shape[0])
     _i32(positions, T, "positions")
     _i32(seq_of_token, T, "seq_of_token")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (nseq, max_blocks)")
     _need(kcache.dtype == qkv.dtype and vcache.dtype == qkv.dtype, "cache and activations differ in type")
-    _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
-          "cache must be (pages, nkv, page_size, d)")
+    _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape[:3] + (vd,),
+          "caches must be (pages, nkv, page_size, d) and (pages, nkv, page_size, vd)")
     _check(lib().gs_qknorm_rope_kv(_p(qkv), c_int(_dt(qkv)), _p(q_weight), _p(k_weight), c_float(eps), _p(cos),
                                    _p(sin), c_int(rotary_dim), c_int(1 if layout == "interleaved" else 0), c_int(max_pos),
                                    _p(positions), _p(seq_of_token),
                                    _p(block_table), c_int(block_table.shape[1]), c_int(page_size), _p(kcache),
                                    _p(vcache), c_int(T), c_int(nh), c_int(nkv), c_int(d),
-                                   c_int(1 if write_kv else 0), _stream()))
+                                   c_int(1 if write_kv else 0), c_int(vd), _p(vcos), _p(vsin), _stream()))
 
 
 def attention_generic(q, q_stride, kcache, vcache, positions, seq_of_token, block_table, page_size, window, scale,
-                      nh, nkv, d, ntok, out: torch.Tensor = None) -> torch.Tensor:
-    """Causal GQA over the paged cache, any sizes; ``q`` rows are ``q_stride`` apart."""
+                      nh, nkv, d, ntok, out: torch.Tensor = None, vd: int = None, chunk: int = None, sink: bool = False,
+                      vcos=None, vsin=None, layout: str = "half") -> torch.Tensor:
+    """Causal GQA over the paged cache, any sizes; ``q`` rows are ``q_stride`` apart.  ``vd``: the width of a value
+    head where it is not ``d``; ``chunk``: a query sees only the keys of its own run of ``chunk`` positions;
+    ``sink``: one more term ``exp(0)`` in the softmax's denominator; ``vcos``, ``vsin``: the cached values are turned
+    by their positions, and a head's sum is turned back by the query's (pairs laid out as ``layout`` says)."""
     _dev(q, kcache, vcache, positions, seq_of_token, block_table, out)
+    vd = d if vd is None else int(vd)
     _need(q.numel() >= (ntok - 1) * q_stride + nh * d if ntok else True, "attention: q is too small")
     _need(kcache.dtype == q.dtype and vcache.dtype == q.dtype, "cache and activations differ in type")
-    _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
-          "cache must be (pages, nkv, page_size, d)")
+    _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape[:3] + (vd,),
+          "caches must be (pages, nkv, page_size, d) and (pages, nkv, page_size, vd)")
+    _value_tables(vcos, vsin, vd)
+    _need(layout in ROPE_LAYOUTS, f"attention: pairs are laid out 'half' or 'interleaved', not {layout!r}")
     _i32(positions, ntok, "positions")
     _i32(seq_of_token, ntok, "seq_of_token")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (nseq, max_blocks)")
     if out is None:
-        out = torch.empty((ntok, nh * d), dtype=q.dtype, device=q.device)
-    _need(out.shape == (ntok, nh * d) and out.dtype == q.dtype, "attention: out has the wrong shape or type")
+        out = torch.empty((ntok, nh * vd), dtype=q.dtype, device=q.device)
+    _need(out.shape == (ntok, nh * vd) and out.dtype == q.dtype, "attention: out has the wrong shape or type")
     _check(lib().gs_attention_generic(_p(q), c_int(q_stride), _p(kcache), _p(vcache), c_int(_dt(q)), _p(positions),
                                       _p(seq_of_token), _p(block_table), c_int(block_table.shape[1]),
                                       c_int(page_size), c_int(window or 0), c_float(scale), _p(out), c_int(ntok),
-                                      c_int(nh), c_int(nkv), c_int(d), _stream()))
+                                      c_int(nh), c_int(nkv), c_int(d), c_int(vd), c_int(chunk or 0),
+                                      c_int(1 if sink else 0), _p(vcos), _p(vsin),
+                                      c_int(1 if layout == "interleaved" else 0), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------- linear attention
+
+_ACTS = {None: 0, "none": 0, "silu": 1}
+_GATES = {"sigmoid": 0, "silu": 1}
+GATED_ACTS = {"silu": 0, "gelu_tanh": 1}
+LINEAR_ATTENTION_MAX_KEY = 256
+
+
+def linear_attention_scan(x, oq: int, ok: int, ov: int, H: int, n: int, m: int, decay, state, q_start, slots, positions,
+                          nseq: int, activation=None, cos=None, sin=None, rotary_dim: int = 0, key_scale: float = 1.0,
+                          out: torch.Tensor = None) -> torch.Tensor:
+    """Linear attention through a fading state: per sequence and head ``S <- decay_h S + k_t v_t^T``, ``o_t = S^T q_t``.
+
+    ``x (T, ld)`` holds q of head h at columns ``[oq + h n, ...)``, k at ``[ok + h n, ...)``, v at ``[ov + h m, ...)``;
+    ``activation`` (None or ``"silu"``) is applied to all three, q and k are turned by ``positions`` over their first
+    ``rotary_dim`` features (half-split pairs, tables ``(P, rotary_dim/2)``), k is multiplied by ``key_scale``.
+    ``state (slots, H, n, m)`` float32 is read and advanced for the sequences' ``slots``.  Returns ``(T, H m)`` float32."""
+    _dev(x, decay, state, q_start, slots, positions, cos, sin, out)
+    _need(x.dim() == 2, "linear_attention: rows (T, ld)")
+    T, ld = x.shape
+    _need(activation in _ACTS, f"linear_attention: activation is None or 'silu', not {activation!r}")
+    _need(decay.dtype == torch.float32 and decay.shape == (H,), "linear_attention: decay must be float32 (H,)")
+    _need(state.dtype == torch.float32 and state.dim() == 4 and state.shape[1:] == (H, n, m),
+          "linear_attention: state must be float32 (slots, H, n, m)")
+    _need(n <= LINEAR_ATTENTION_MAX_KEY, f"linear_attention: keys of {n} features, the kernel holds up to {LINEAR_ATTENTION_MAX_KEY}")
+    _i32(q_start, nseq + 1, "q_start")
+    _i32(slots, nseq, "slots")
+    _i32(positions, T, "positions")
+    max_pos = 0
+    if rotary_dim:
+        _need(cos is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape
+              and cos.dim() == 2 and cos.shape[1] == rotary_dim // 2, "linear_attention: tables must be float32 (P, rotary_dim/2)")
+        max_pos = cos.shape[0]
+    if out is None:
+        out = torch.empty((T, H * m), dtype=torch.float32, device=x.device)
+    _need(out.shape == (T, H * m) and out.dtype == torch.float32, "linear_attention: out must be float32 (T, H m)")
+    _check(lib().gs_linear_attention_scan(_p(x), c_int(_dt(x)), c_int(ld), c_int(oq), c_int(ok), c_int(ov),
+                                          c_int(_ACTS[activation]), _p(cos) if rotary_dim else None,
+                                          _p(sin) if rotary_dim else None, c_int(rotary_dim), c_int(max_pos),
+                                          c_float(key_scale), _p(decay), _p(state), _p(q_start), _p(slots), _p(positions),
+                                          _p(out), c_int(nseq), c_int(H), c_int(n), c_int(m), _stream()))
+    return out
+
+
+def gated_outnorm(o, gate_rows, og: int, weight, eps: float, H: int, m: int, joint: bool, gate: str, out_dtype) -> torch.Tensor:
+    """``o (T, H m)`` float32 normed (``joint``: all heads as one row, times ``weight``; else each head by its own root
+    mean square) and multiplied by ``sigmoid`` or ``silu`` of the gate, which stands in ``gate_rows (T, ldg)`` from
+    column ``og`` on.  Returns ``(T, H m)`` in ``out_dtype``."""
+    _dev(o, gate_rows, weight)
+    T = o.shape[0]
+    _need(o.dtype == torch.float32 and o.shape == (T, H * m), "gated_outnorm: o must be float32 (T, H m)")
+    _need(gate_rows.dim() == 2 and gate_rows.shape[0] == T and gate_rows.dtype == out_dtype,
+          "gated_outnorm: the gate's rows are (T, ldg) in the result's type")
+    _need(weight is None or (weight.dtype == torch.float32 and weight.shape == (H * m,)), "gated_outnorm: weight must be float32 (H m,)")
+    _need(gate in _GATES, f"gated_outnorm: the gate is 'sigmoid' or 'silu', not {gate!r}")
+    out = torch.empty((T, H * m), dtype=out_dtype, device=o.device)
+    _check(lib().gs_gated_outnorm(_p(o), _p(gate_rows), c_int(_dt(gate_rows)), c_int(gate_rows.shape[1]), c_int(og),
+                                  _p(weight), c_float(eps), c_int(1 if joint else 0), c_int(_GATES[gate]), _p(out),
+                                  c_int(_dt(out)), c_int(T), c_int(H), c_int(m), _stream()))
+    return out
+
+
+def add_rmsnorm_pair(res, d1, d2, w1, w2, eps: float, out_dtype):
+    """``res += d1 + d2`` (each where given), then ``(rmsnorm(res) * w1, rmsnorm(res) * w2)``; ``w2`` None: one result."""
+    _dev(res, d1, d2, w1, w2)
+    _need(res.dtype == torch.float32 and res.dim() == 2, "add_rmsnorm_pair: the residual stream is float32 (T, H)")
+    T, H = res.shape
+    for w in (w1, w2):
+        _need(w is None or (w.dtype == torch.float32 and w.shape == (H,)), "add_rmsnorm_pair: weights must be float32 (H,)")
+    _need(w1 is not None, "add_rmsnorm_pair: a first weight")
+    ds = [d for d in (d1, d2) if d is not None]
+    for d in ds:
+        _need(d.shape == res.shape and d.dtype == ds[0].dtype, "add_rmsnorm_pair: deltas have the stream's shape and one type")
+    out1 = torch.empty((T, H), dtype=out_dtype, device=res.device)
+    out2 = torch.empty((T, H), dtype=out_dtype, device=res.device) if w2 is not None else None
+    _check(lib().gs_add_rmsnorm_pair(_p(res), _p(ds[0]) if ds else None, _p(ds[1]) if len(ds) > 1 else None,
+                                     c_int(_dt(ds[0]) if ds else _dt(out1)), _p(w1), _p(w2), c_float(eps), _p(out1),
+                                     _p(out2), c_int(_dt(out1)), c_int(T), c_int(H), _stream()))
+    return out1, out2
+
+
+def scaled_sum(a, sa: float, b, sb: float, out_dtype) -> torch.Tensor:
+    """``sa * a + sb * b`` in float32, rounded once to ``out_dtype``; ``a`` and ``b`` of one shape and type."""
+    _dev(a, b)
+    _need(a.shape == b.shape and a.dtype == b.dtype, "scaled_sum: operands of one shape and type")
+    out = torch.empty(a.shape, dtype=out_dtype, device=a.device)
+    _check(lib().gs_scaled_sum(_p(a), c_float(sa), _p(b), c_float(sb), c_int(_dt(a)), _p(out), c_int(_dt(out)),
+                               c_long(a.numel()), _stream()))
+    return out
+
+
+def gated_act(x, bias, activation: str, out_dtype) -> torch.Tensor:
+    """``x (T, 2F)`` = gate | up, ``bias (2F,)`` float32 or None -> ``act(gate + b) * (up + b) (T, F)`` in ``out_dtype``."""
+    _dev(x, bias)
+    _need(x.dim() == 2 and x.shape[1] % 2 == 0, "gated_act: rows hold gate and up side by side")
+    T, F2 = x.shape
+    F = F2 // 2
+    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (F2,)), "gated_act: bias must be float32 (2F,)")
+    _need(activation in GATED_ACTS, f"gated_act: the activation is one of {sorted(GATED_ACTS)}, not {activation!r}")
+    out = torch.empty((T, F), dtype=out_dtype, device=x.device)
+    _check(lib().gs_gated_act(_p(x), c_int(_dt(x)), _p(bias), _p(out), c_int(_dt(out)), c_int(T), c_int(F),
+                              c_int(GATED_ACTS[activation]), _stream()))
     return out
 
 

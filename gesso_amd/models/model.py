@@ -30,6 +30,9 @@ def tensor_table(spec: ModelSpec) -> Dict[str, TensorSpec]:
     put(spec.names["embed"], TensorSpec((spec.vocab, spec.hidden), TABLE))
     for local, ts in part_class("norm", spec.final_norm).tensor_specs(spec.final_norm).items():
         put(spec.names["final_norm." + local], ts)
+    if spec.embed_norm is not None:
+        for local, ts in part_class("norm", spec.embed_norm).tensor_specs(spec.embed_norm).items():
+            put(spec.names["embed_norm." + local], ts)
     if not spec.tie_embeddings:
         put(spec.names["head"], TensorSpec((spec.vocab, spec.hidden), MATRIX))
     for i, b in enumerate(spec.blocks):
@@ -53,6 +56,7 @@ class Model:
         self.rt = rt
         self.blocks = [build("block", b, rt) for b in spec.blocks]
         self.final_norm = build("norm", spec.final_norm, rt)
+        self.embed_norm = build("norm", spec.embed_norm, rt) if spec.embed_norm is not None else None
         self.embed = None
         self.head = None
 
@@ -71,13 +75,17 @@ class Model:
         self.head = self.rt.prepare(self.embed if s.tie_embeddings else tensors[s.names["head"]])
         self.final_norm.bind({k: tensors[s.names["final_norm." + k]]
                               for k in part_class("norm", s.final_norm).tensor_specs(s.final_norm)})
+        if self.embed_norm is not None:
+            self.embed_norm.bind({k: tensors[s.names["embed_norm." + k]]
+                                  for k in part_class("norm", s.embed_norm).tensor_specs(s.embed_norm)})
         for b, block in zip(s.blocks, self.blocks):
             local = {k: tensors[b.names[k]] for k in part_class("block", b).tensor_specs(b)}
             block.bind(local)
 
     @property
     def graph_safe(self) -> bool:
-        return all(getattr(b, "graph_safe", False) for b in self.blocks) and getattr(self.final_norm, "graph_safe", False)
+        norms = [self.final_norm] + ([self.embed_norm] if self.embed_norm is not None else [])
+        return all(getattr(b, "graph_safe", False) for b in self.blocks) and all(getattr(n, "graph_safe", False) for n in norms)
 
     def forward(self, ctx) -> Optional[torch.Tensor]:
         """Run the tokens of ``ctx`` through every scheduled block; float32 logits at ``ctx.want_rows``."""
@@ -130,6 +138,10 @@ class Model:
 
     def _embed(self, ctx, order, scale):
         ops, rt = self.rt.ops, self.rt
+        if self.embed_norm is not None:
+            # the embedding rows are normed before the first block: the stream starts from the normed rows (float32)
+            raw = ops.embed(ctx.token_ids, self.embed, scale=scale)
+            return ResidualStream(self.embed_norm.add_norm(ResidualStream(raw), out_dtype=torch.float32))
         if rt.fused:
             ssq = torch.empty((ctx.T, 1), dtype=torch.float32, device=rt.device)
             first = getattr(order[0], "first_norm", None) if order else None

@@ -41,15 +41,27 @@ class Attention(Part):
             raise ValueError("query heads must be a multiple of key heads")
         self.position = build("position", spec.position, rt)
         self.scale = spec.scale if spec.scale is not None else 1.0 / math.sqrt(spec.head_dim)
+        # a value head's width; what the kernels written for plain causal attention do not know: values of another
+        # width than the keys, runs of positions, a sink term, values cached turned
+        self.value_dim = spec.head_dim if getattr(spec, "value_dim", None) is None else int(spec.value_dim)
+        self.chunk = getattr(spec, "chunk", None)
+        self.sink = bool(getattr(spec, "sink", False))
+        vp = getattr(spec, "value_position", None)
+        self.value_position = build("position", vp, rt) if vp is not None else None
+        if self.value_position is not None and self.value_position.rotary_dim != self.value_dim:
+            raise ValueError("values are turned over their whole width")
+        self.plain = (self.value_dim == spec.head_dim and not self.chunk and not self.sink
+                      and self.value_position is None)
 
     @staticmethod
     def tensor_specs(spec):
         H, nh, nkv, d = spec.hidden, spec.n_heads, spec.n_kv_heads, spec.head_dim
+        vd = d if getattr(spec, "value_dim", None) is None else spec.value_dim
         out = {"q_proj.weight": TensorSpec((nh * d, H), MATRIX), "k_proj.weight": TensorSpec((nkv * d, H), MATRIX),
-               "v_proj.weight": TensorSpec((nkv * d, H), MATRIX), "out_proj.weight": TensorSpec((H, nh * d), MATRIX)}
+               "v_proj.weight": TensorSpec((nkv * vd, H), MATRIX), "out_proj.weight": TensorSpec((H, nh * vd), MATRIX)}
         if spec.bias:
             out.update({"q_proj.bias": TensorSpec((nh * d,), VECTOR), "k_proj.bias": TensorSpec((nkv * d,), VECTOR),
-                        "v_proj.bias": TensorSpec((nkv * d,), VECTOR), "out_proj.bias": TensorSpec((H,), VECTOR)})
+                        "v_proj.bias": TensorSpec((nkv * vd,), VECTOR), "out_proj.bias": TensorSpec((H,), VECTOR)})
         if spec.qk_norm is not None:
             out.update({"q_norm.weight": TensorSpec((d,), VECTOR, "one_plus_normal"),
                         "k_norm.weight": TensorSpec((d,), VECTOR, "one_plus_normal")})
@@ -57,7 +69,9 @@ class Attention(Part):
 
     @staticmethod
     def cache_need(spec):
-        return PagedKV(spec.n_kv_heads, spec.head_dim, spec.window)
+        vd = getattr(spec, "value_dim", None)
+        return PagedKV(spec.n_kv_heads, spec.head_dim, spec.window, value_dim=None if vd in (None, spec.head_dim) else vd,
+                       chunk=getattr(spec, "chunk", None))
 
     def bind(self, tensors):
         ws = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
@@ -72,10 +86,14 @@ class Attention(Part):
         self.q_norm = tensors.get("q_norm.weight")
         self.k_norm = tensors.get("k_norm.weight")
 
-    def forward(self, x, ctx, cache):
+    takes_out_dtype = True
+
+    def forward(self, x, ctx, cache, out_dtype=None):
         q, q_stride = self.project_in(x, ctx, cache)
         with self.rt.stage("attn_core"):
             o = self.attend(q, q_stride, ctx, cache)
+        if out_dtype is not None:
+            return self.rt.linear(o, self.wo, self.bo, out_dtype=out_dtype)
         return self.rt.project(o, self.wo, self.bo)
 
     # ------------------------------------------------------------------ the mixer's inner steps
@@ -90,15 +108,17 @@ class Attention(Part):
         layout = getattr(pos, "layout", "half")
         with rt.stage("attn_proj"):
             qkv = rt.linear(x, self.wqkv, self.bqkv)      # a lazy norm goes through as it is where the product takes it
-        stride = (nh + 2 * nkv) * d
-        if (rt.fused and ctx.all_single and cache.k.dtype == torch.bfloat16 and qkv.dtype == torch.bfloat16
+        stride = (nh + nkv) * d + nkv * self.value_dim
+        vp = self.value_position
+        if (self.plain and rt.fused and ctx.all_single and cache.k.dtype == torch.bfloat16 and qkv.dtype == torch.bfloat16
                 and cache.page_size >= 2 and (self.q_norm is None) == (self.k_norm is None) and layout == "half"
                 and ops.attention_decode_raw_supports(nh, nkv, d, pos.rotary_dim)):
             return RawQKV(qkv, self.q_norm, self.k_norm, eps, pos), stride
         with rt.stage("attn_headnorm_rope"):
             ops.qknorm_rope_kv(qkv, self.q_norm, self.k_norm, eps, pos.cos, pos.sin, pos.rotary_dim, ctx.positions,
                                ctx.seq_of_token, cache.block_table, cache.page_size, cache.k, cache.v, nh, nkv, d,
-                               write_kv=cache.write, layout=layout)
+                               write_kv=cache.write, layout=layout, vd=self.value_dim,
+                               vcos=None if vp is None else vp.cos, vsin=None if vp is None else vp.sin)
         return qkv, stride
 
     def _single(self, q, q_stride, cache, ctx, nseq, out):
@@ -141,6 +161,8 @@ class Attention(Part):
         (or, of single tokens, would split their keys over blocks by the longest sequence), and is not to be recorded."""
         s, rt, ops = self.spec, self.rt, self.rt.ops
         nh, nkv, d = s.n_heads, s.n_kv_heads, s.head_dim
+        if not self.plain:
+            return False
         lead = 0
         while lead < len(q_lens) and q_lens[lead] == 1:
             lead += 1
@@ -186,6 +208,16 @@ class Attention(Part):
                                           cache.page_size, window, self.scale, nh, nkv, d, ctx.T, out=out,
                                           key_splits=halves)
 
+    def _attend_general(self, q, q_stride, ctx, cache) -> torch.Tensor:
+        """Attention with values of their own width, runs of positions, a sink term or turned values: ``(T, nh * vd)``."""
+        s, ops, vp = self.spec, self.rt.ops, self.value_position
+        layout = getattr(vp, "layout", "half") if vp is not None else "half"
+        return ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token, cache.block_table,
+                                     cache.page_size, s.window, self.scale, s.n_heads, s.n_kv_heads, s.head_dim, ctx.T,
+                                     vd=self.value_dim, chunk=self.chunk, sink=self.sink,
+                                     vcos=None if vp is None else vp.cos, vsin=None if vp is None else vp.sin,
+                                     layout=layout)
+
     def attend(self, q, q_stride, ctx, cache) -> torch.Tensor:
         """Causal attention of this step's queries over the paged cache; ``(T, nh * d)``.
 
@@ -194,6 +226,8 @@ class Attention(Part):
         """
         s, rt, ops = self.spec, self.rt, self.rt.ops
         nh, nkv, d, window = s.n_heads, s.n_kv_heads, s.head_dim, s.window
+        if not self.plain:
+            return self._attend_general(q, q_stride, ctx, cache)
         out = True if rt.rows_tiled(nh * d) else None
         if isinstance(q, RawQKV):
             return self._single(q, q_stride, cache, ctx, ctx.nseq, out)

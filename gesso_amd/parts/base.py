@@ -14,7 +14,8 @@ Interfaces (duck-typed; the classes below are convenient bases):
                   ``cos``, ``sin`` (``(max_position, rotary_dim/2)`` float32), ``rotary_dim`` and ``layout``
                   (``"half"``: pairs ``(i, i + rotary_dim/2)``, ``"interleaved"``: ``(2i, 2i + 1)``);
                   or ``rotary_dim == 0`` for none
-* mixer           ``tensor_specs(spec)``, ``cache_need(spec) -> PagedKV | SlotState | None``,
+* mixer           ``tensor_specs(spec)``, ``cache_need(spec) -> PagedKV | SlotState | None`` or a tuple of these
+                  (a mixer made of several, each with a cache of its own: ``cache`` is then a tuple of views),
                   ``bind(tensors)``, ``forward(x, ctx, cache) -> (T, hidden)``
 * feed-forward    ``tensor_specs(spec)``, ``bind(tensors)``, ``forward(x, ctx) -> (T, hidden)``
 * block           ``tensor_specs(spec)``, ``cache_need(spec)``, ``bind``,
@@ -50,12 +51,24 @@ class PagedKV:
     token and derives both from it).
 
     ``window``: only the last ``window`` tokens are ever read again (None = all of them).
+    ``chunk``: positions are cut into runs of ``chunk`` from 0 on and a token reads only its own run, so the runs
+    before the newest token's are never read again (None = no such cut).
     """
 
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None
+    chunk: Optional[int] = None
+
+    def first_needed(self, length: int) -> int:
+        """The oldest position that the token after ``length`` cached ones can read."""
+        first = 0
+        if self.window is not None:
+            first = max(first, length - self.window + 1)
+        if self.chunk is not None:
+            first = max(first, length - length % self.chunk)
+        return first
 
     @property
     def value_width(self) -> int:

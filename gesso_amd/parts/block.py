@@ -117,5 +117,36 @@ class OutNormBlock(PreNormBlock):
         return False
 
 
+class ParallelBlock(PreNormBlock):
+    """``h += mixer(norm_a(h)) + ffn(norm_b(h))``: both sub-layers read the stream as it enters the block, each
+    through its own norm.  One kernel adds what the block before left (its two results) and norms the row for both
+    readers; the block's own two results stay beside the stream for whoever norms it next."""
+
+    def forward(self, stream, ctx, cache):
+        rt, ops = self.rt, self.rt.ops
+        held = stream.pending if isinstance(stream.pending, tuple) else (stream.pending, None)
+        with rt.stage("norm"):
+            second = self.ffn_norm if self.ffn is not None else None
+            x1, x2 = ops.add_rmsnorm_pair(stream.res, held[0], held[1], self.mixer_norm.weight,
+                                          None if second is None else second.weight, self.mixer_norm.spec.eps, rt.dtype)
+        stream.pending = stream.ssq = stream.xs = stream.xs_for = stream.normed = stream.rows = None
+        with rt.stage(getattr(self.mixer, "stage", "mixer")):
+            a = rt.dense(self.mixer.forward(x1, ctx, cache))
+        b = None
+        if self.ffn is not None:
+            with rt.stage(getattr(self.ffn, "stage", "ffn")):
+                b = rt.dense(self.ffn.forward(x2, ctx))
+        stream.pending = (a, b)
+
+    @property
+    def first_norm(self):
+        return None                 # the block norms the stream itself, twice in one pass
+
+    @property
+    def portions_recordable(self) -> bool:
+        return False
+
+
 register("block", "prenorm", PreNormBlock)
+register("block", "parallel", ParallelBlock)
 register("block", "outnorm", OutNormBlock)

@@ -1,0 +1,53 @@
+"""Gated feed-forward with a choice of activation and optional biases:
+``W_down (act(W_gate x + b_gate) * (W_up x + b_up)) + b_down``; ``act`` is silu or the tanh form of gelu.
+
+W_gate and W_up are laid side by side at load so that one product feeds both (as :mod:`gesso_amd.parts.swiglu` does);
+biases, activation and the product of the two halves are one pass in float32 over the product's rows.
+"""
+from __future__ import annotations
+
+import torch
+
+from .base import MATRIX, VECTOR, Part, TensorSpec
+from .registry import register
+
+
+class GatedMLP(Part):
+    graph_safe = True
+    stage, out_stage = "dense_ffn", "ffn_down"
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        if spec.activation not in rt.ops.GATED_ACTS:
+            raise ValueError(f"activation {spec.activation!r}; the kernel has {sorted(rt.ops.GATED_ACTS)}")
+
+    @staticmethod
+    def tensor_specs(spec):
+        H, F = spec.hidden, spec.intermediate
+        out = {"gate.weight": TensorSpec((F, H), MATRIX), "up.weight": TensorSpec((F, H), MATRIX),
+               "down.weight": TensorSpec((H, F), MATRIX)}
+        if spec.bias:
+            out.update({"gate.bias": TensorSpec((F,), VECTOR), "up.bias": TensorSpec((F,), VECTOR),
+                        "down.bias": TensorSpec((H,), VECTOR)})
+        return out
+
+    def bind(self, tensors):
+        g, u = tensors["gate.weight"], tensors["up.weight"]
+        if g.dtype != u.dtype:
+            g, u = g.float(), u.float()
+        self.w_gu = self.rt.prepare(torch.cat([g, u], 0).contiguous(), unit=g.shape[0])
+        self.w_down = self.rt.prepare(tensors["down.weight"])
+        self.b_gu = self.b_down = None
+        if self.spec.bias:
+            self.b_gu = torch.cat([tensors["gate.bias"], tensors["up.bias"]], 0).contiguous()
+            self.b_down = tensors["down.bias"]
+
+    def forward(self, x, ctx):
+        rt = self.rt
+        with rt.stage("ffn_gateup"):
+            gu = rt.linear(rt.dense(x), self.w_gu)
+            a = rt.ops.gated_act(gu, self.b_gu, self.spec.activation, rt.dtype)
+        return rt.linear(a, self.w_down, self.b_down)
+
+
+register("ffn", "gated_mlp", GatedMLP)

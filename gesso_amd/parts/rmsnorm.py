@@ -1,4 +1,5 @@
-"""RMSNorm: ``y = x / sqrt(mean(x^2) + eps) * w`` over the last axis, eps inside the root, no +1.
+"""RMSNorm: ``y = x / sqrt(mean(x^2) + eps) * w`` over the last axis, eps inside the root.  A spec with an ``offset``
+stores its weight around zero: ``w = offset + stored`` is formed once, in float32, when the weight is bound.
 
 Reference: ``src/Operators/cpu.jl:293-312``.  The kernel folds the residual add that precedes
 the norm into the same pass, as the reference's seam does (``src/Inference/Inference.jl:1936-1939``).
@@ -63,7 +64,9 @@ class ResidualStream:
     def flush(self, rt) -> None:
         """Add what is pending, if a norm has not done so."""
         if self.pending is not None:
-            rt.ops.residual_add(self.res, self.pending)
+            for delta in (self.pending if isinstance(self.pending, tuple) else (self.pending,)):
+                if delta is not None:
+                    rt.ops.residual_add(self.res, delta)      # (a parallel block leaves two results)
             self.pending, self.ssq = None, None
             self.xs = self.xs_for = self.normed = self.rows = None
 
@@ -82,28 +85,32 @@ class RMSNorm(Part):
 
     @staticmethod
     def tensor_specs(spec):
-        return {"weight": TensorSpec((spec.size,), VECTOR, "one_plus_normal")}
+        around_zero = getattr(spec, "offset", 0.0) != 0.0
+        return {"weight": TensorSpec((spec.size,), VECTOR, "normal" if around_zero else "one_plus_normal")}
 
     def bind(self, tensors):
-        self.weight = tensors["weight"]
+        offset = float(getattr(self.spec, "offset", 0.0))
+        self.weight = tensors["weight"] if offset == 0.0 else (tensors["weight"].float() + offset).contiguous()
 
     @property
     def row_weight(self):
         """``norm(x) = inv_rms(x) * (x * row_weight)``: what lets a producer pre-weight the rows for this norm."""
         return self.weight if self.rt.dtype == torch.bfloat16 else None
 
-    def add_norm(self, stream: ResidualStream, rows=None, out=None):
+    def add_norm(self, stream: ResidualStream, rows=None, out=None, out_dtype=None):
         """Add what is pending to the stream, then norm it (only ``rows`` of it when given).
 
         While a decode step is recorded with fused kernels, and the stream's sums of squares are at
         hand, the norm is not run: a :class:`~gesso_amd.kernels.ops.LazyNorm` goes to the product that
         follows, which norms on the fly.
         """
+        if isinstance(stream.pending, tuple):
+            stream.flush(self.rt)
         if self.rt.fused and rows is None and stream.pending is None and stream.ssq is not None:
             mine = stream.xs_for is self
             return self.rt.ops.LazyNorm(stream.res, stream.ssq, self.weight, self.spec.eps, self.rt.dtype,
                                         xs=stream.xs if mine else None, ready=stream.normed if mine else None)
-        y = self.rt.ops.add_rmsnorm(stream.res, stream.pending, self.weight, self.spec.eps, self.rt.dtype,
+        y = self.rt.ops.add_rmsnorm(stream.res, stream.pending, self.weight, self.spec.eps, out_dtype or self.rt.dtype,
                                     rows=rows, out=out)
         if rows is None:
             stream.pending = None

@@ -87,6 +87,49 @@ class ScaledRope(Part):
             self.cos, self.sin = rt.shared(key, make)
 
 
+def stretched_rope_tables(spec):
+    """cos and sin tables of a :class:`~gesso_amd.config.spec.StretchedRopeSpec` (see there for the rule): a pair keeps
+    its frequency, gets it divided by ``factor``, or a blend of both, by where its wavelength stands against
+    ``original / high`` and ``original / low``.  float64 on the host, stored as float32."""
+    import math
+    dims, theta = spec.rotary_dim, float(spec.theta)
+    freq = [theta ** (-2.0 * i / dims) for i in range(dims // 2)]
+    if spec.factor is not None:
+        factor, low, high, original = float(spec.factor), float(spec.low), float(spec.high), float(spec.original)
+        for i, f in enumerate(freq):
+            wavelength = 2.0 * math.pi / f
+            if wavelength > original / low:
+                freq[i] = f / factor
+            elif wavelength >= original / high:
+                s = (original / wavelength - low) / (high - low)
+                freq[i] = (1.0 - s) * f / factor + s * f
+    ang = torch.arange(spec.max_position, dtype=torch.float64)[:, None] * torch.tensor(freq, dtype=torch.float64)[None, :]
+    return torch.cos(ang).to(torch.float32), torch.sin(ang).to(torch.float32)
+
+
+class StretchedRope(Part):
+    """Rotation with frequencies stretched by wavelength: the same three attributes as :class:`Rope`, other tables."""
+
+    graph_safe = True
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        if spec.rotary_dim % 2 or not 0 < spec.rotary_dim <= spec.head_dim:
+            raise ValueError(f"rotary_dim {spec.rotary_dim} must be even and within the head width {spec.head_dim}")
+        self.rotary_dim = spec.rotary_dim
+        self.layout = spec.layout
+        if self.layout not in rt.ops.ROPE_LAYOUTS:
+            raise ValueError(f"rotation pairs are laid out 'half' or 'interleaved', not {self.layout!r}")
+
+        def make():
+            cos, sin = stretched_rope_tables(spec)
+            return cos.to(rt.device), sin.to(rt.device)
+
+        key = ("stretched_rope", spec.rotary_dim, float(spec.theta), spec.max_position, spec.factor, float(spec.original),
+               float(spec.low), float(spec.high))
+        self.cos, self.sin = rt.shared(key, make)
+
+
 class NoPosition(Part):
     graph_safe = True
     rotary_dim = 0
@@ -97,4 +140,5 @@ class NoPosition(Part):
 
 register("position", "rope", Rope)
 register("position", "scaled_rope", ScaledRope)
+register("position", "stretched_rope", StretchedRope)
 register("position", "none", NoPosition)
