@@ -9,6 +9,7 @@ import sys
 import numpy as np
 import torch
 
+import plain_fazezen
 import plain_lfm2
 import plain_makuzen
 
@@ -19,9 +20,9 @@ TRACE_RUN = os.path.join(ROOT, "bin", "trace_run")
 def plain_logits(model_dir: str, ids, rounded: bool = False) -> np.ndarray:
     """(T, V) float64 logits of the whole sequence by the plain implementation; ``rounded``: with its activations
     rounded to bfloat16 wherever a pipeline with bfloat16 activations stores one."""
-    # each architecture has its own plain implementation; both read a folder and offer forward(cfg, w, ids, store=)
+    # each architecture has its own plain implementation; all read a folder and offer forward(cfg, w, ids, store=)
     with open(os.path.join(model_dir, "config.json"), encoding="utf-8") as f:
-        P = plain_makuzen if json.load(f).get("architecture") == "Makuzen" else plain_lfm2
+        P = {"Makuzen": plain_makuzen, "Fazezen": plain_fazezen}.get(json.load(f).get("architecture"), plain_lfm2)
     cfg = P.read_config(model_dir)
     w = P.read_weights(model_dir, torch.float64)
     return P.forward(cfg, w, list(ids), **({"store": P.to_bfloat16} if rounded else {})).numpy()
