@@ -51,9 +51,18 @@ def weight_bytes(engine) -> int:
     seen, n = set(), 0
     m = engine.model
     tensors = [m.head, m.final_norm.weight]
+    def of(part):
+        out = []
+        for v in (vars(part).values() if part is not None else ()):
+            if isinstance(v, torch.Tensor):
+                out.append(v)
+            elif hasattr(v, "spec") and hasattr(v, "rt") and not hasattr(v, "cos"):      # a part inside a part
+                out += of(v)
+        return out
+
     for b in m.blocks:
         for part in (b.mixer_norm, b.mixer, b.ffn_norm, b.ffn):
-            tensors += [v for v in vars(part).values() if isinstance(v, torch.Tensor)]
+            tensors += of(part)
     for t in tensors:
         if t.data_ptr() not in seen:
             seen.add(t.data_ptr())
@@ -376,6 +385,65 @@ def makuzen_workload(steps: int = 64, warmup: int = 8, sizes=("1024", "2048"), o
     return out
 
 
+FAZEZEN_SIZES = {
+    # six layers of linear attention through a fading state and two pairs (attention within runs beside retention), in
+    # the places where LFM2's first eight layers have convolutions and attention; the feed-forward as wide as LFM2's
+    "1024": dict(width=1024, heads=16, dim=64, vdim=64, left=(16, 4, 64, 64), right=(8, 64, 128), chunk=512, ff=4608,
+                 vocab=65536, beside="350m"),
+    "2048": dict(width=2048, heads=16, dim=128, vdim=128, left=(32, 8, 64, 64), right=(16, 64, 128), chunk=1024, ff=8192,
+                 vocab=65536, beside="1.2b"),
+}
+
+
+def fazezen_config(size: str, max_position: int = 4096):
+    from gesso_amd.config import (ChunkedAttentionConfig, DenseConfig, FazezenConfig, FazezenLayer, LightningConfig,
+                                  ParallelConfig, RetentionConfig, Rotation, Stretch)
+    z = FAZEZEN_SIZES[size]
+    H = z["heads"]
+    light = LightningConfig(H, z["dim"], z["vdim"], tuple(1.0 - 2.0 ** (-3 - 6 * h / (H - 1)) for h in range(H)))
+    nh, nkv, d, vd = z["left"]
+    rh, rn, rm = z["right"]
+    pair = ParallelConfig(
+        ChunkedAttentionConfig(nh, nkv, d, vd, d ** -0.5, Rotation(1e6, d, Stretch(4.0, 1.0, 4.0, 2048.0)), z["chunk"]),
+        RetentionConfig(rh, rn, rm, tuple(1.0 - 2.0 ** (-5 - 5 * h / (rh - 1)) for h in range(rh)), Rotation(1e6, rn)), 1.2, 0.9)
+    layers = tuple(FazezenLayer("parallel", pair, DenseConfig(z["ff"])) if i in (2, 5) else
+                   FazezenLayer("lightning", light, DenseConfig(z["ff"])) for i in range(8))
+    return FazezenConfig(vocab=z["vocab"], width=z["width"], layers=layers, norm_eps=1e-5, max_position=max_position)
+
+
+def fazezen_workload(steps: int = 64, warmup: int = 8, sizes=("1024", "2048"), only: str = "", batches=(8, 64)) -> dict:
+    """Fazezen (linear attention through a fading state, pairs of attention within runs beside retention, blocks whose
+    sub-layers read one stream) at two sets of layer sizes, beside LFM2 of the same width and depth: a 2,048-token
+    prompt in one step, and decode steps at 512-token prompts."""
+    import dataclasses
+    from gesso_amd import Engine
+    from gesso_amd.parts import RuntimeOptions
+    out = {"metric": "Fazezen beside LFM2 at equal width and depth: prefill and decode tok/s", "unit": "tok/s", "dtype": "bf16",
+           "data": "synthetic: uniform random token ids, random weights N(0, 0.02)", "sizes": {}}
+    for size in sizes:
+        z = FAZEZEN_SIZES[size]
+        lfm = model_config(z["beside"])
+        lfm = dataclasses.replace(lfm, num_hidden_layers=8, layer_types=lfm.layer_types[:8])
+        row = {}
+        for name, cfg in (("fazezen", fazezen_config(size)), ("lfm2", lfm)):
+            if only and only != name:
+                continue
+            engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", page_size=16, max_context=4096,
+                                        max_tokens=max(batches) * (512 + steps + warmup + 32) + 4096, num_slots=max(batches) + 1,
+                                        options=RuntimeOptions(tune_library=True))
+            sec = prefill_run(engine, cfg, 2048)
+            r = {"prefill_tok_s": round(2048 / sec, 1), "prefill_ms": round(sec * 1e3, 3), "weights_gb": round(weight_bytes(engine) / 1e9, 3)}
+            for b in batches:
+                dt, _ = decode_run(engine, cfg, b, 512, steps, warmup, seed=40 + b)
+                r[f"decode_b{b}_tok_s"] = round(b * steps / dt, 1)
+                r[f"decode_b{b}_ms"] = round(dt / steps * 1e3, 4)
+            row[name] = r
+            del engine
+            torch.cuda.empty_cache()
+        out["sizes"][size] = row
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -395,11 +463,13 @@ def main() -> int:
     ap.add_argument("--launched-portions", action="store_true", help="launch the steps with prompt portions kernel by kernel instead of "
                     "replaying recordings of them (the prefill of the default line, --workload serve)")
     ap.add_argument("--token-budget", type=int, default=4096, help="--workload serve: the most tokens a step holds")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages", "makuzen"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages", "makuzen", "fazezen"],
                     help="decode: the default line; serve: continuous batching at LFM2-350M sizes; long: LFM2-2.6B "
                          "sizes at a context of 32,768; gemm: the products of a 2,048-token prompt, ours beside the vendor's; "
                          "stages: the decode step stage by stage; makuzen: the Makuzen design at two sets of layer sizes "
-                         "beside LFM2 of equal width and depth")
+                         "beside LFM2 of equal width and depth; fazezen: the same for the Fazezen design")
+    ap.add_argument("--fazezen-sizes", default="1024,2048", help="--workload fazezen: which of its sizes")
+    ap.add_argument("--fazezen-only", default="", choices=["", "fazezen", "lfm2"], help="--workload fazezen: one of the two models (for profiling)")
     ap.add_argument("--makuzen-sizes", default="1024,2048", help="--workload makuzen: which of its sizes")
     ap.add_argument("--makuzen-only", default="", choices=["", "makuzen", "lfm2"], help="--workload makuzen: one of the two models (for profiling)")
     args = ap.parse_args()
@@ -413,6 +483,10 @@ def main() -> int:
         if args.workload == "makuzen":
             print(json.dumps(makuzen_workload(min(args.steps, 64), min(args.warmup, 8), tuple(args.makuzen_sizes.split(",")),
                                               args.makuzen_only)))
+            return 0
+        if args.workload == "fazezen":
+            print(json.dumps(fazezen_workload(min(args.steps, 64), min(args.warmup, 8), tuple(args.fazezen_sizes.split(",")),
+                                              args.fazezen_only)))
             return 0
         if args.workload == "serve":
             print(json.dumps(serve_workload(record=not args.launched_portions, tune=not args.no_tune, budget=args.token_budget)))

@@ -14,7 +14,8 @@
 // rg, rg + 4, ... of column jl in registers; the four partial sums of a column's output are neighbours in a
 // wavefront.  A step's tokens come through LDS eight at a time.  The sums run in one fixed order per output, whatever
 // the step's cut: a sequence fed whole, in portions or token by token leaves the same state and outputs, bit for bit.
-// A step of single tokens is the same kernel with one token a block.
+// A step of single tokens is the same kernel with one token a block.  With `below` > 0 only the sequences that bring
+// fewer tokens than that are taken: the longer ones go to the kernel on the matrix cores (linear_attention_mfma.hip).
 //
 // gated_outnorm: the heads' outputs of a token, normed in float32 (all heads as one row with a weight, or each head by
 // its own root mean square, no weight) and multiplied by sigmoid or silu of a gate row.
@@ -31,7 +32,8 @@ linear_attention_scan_kernel(const TI* __restrict__ x, int ld, int oq, int ok, i
                              const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rd, float key_scale,
                              const float* __restrict__ decay, float* __restrict__ state,
                              const int* __restrict__ q_start, const int* __restrict__ slots,
-                             const int* __restrict__ positions, float* __restrict__ out, int H, int n, int m) {
+                             const int* __restrict__ positions, float* __restrict__ out, int H, int n, int m,
+                             int below) {
   constexpr int NMAX = 4 * RMAX;
   __shared__ float qs[LA_TB][NMAX];
   __shared__ float ks[LA_TB][NMAX];
@@ -39,7 +41,7 @@ linear_attention_scan_kernel(const TI* __restrict__ x, int ld, int oq, int ok, i
   const int seq = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * LA_COLS;
   const int tid = threadIdx.x, rg = tid & 3, jl = tid >> 2, j = j0 + jl;
   const int t0 = q_start[seq], t1 = q_start[seq + 1];
-  if (t1 <= t0) return;
+  if (t1 <= t0 || (below > 0 && t1 - t0 >= below)) return;      // (longer sequences are another kernel's)
   const float d = decay[h];
   float* S = state + (((size_t)slots[seq] * H + h) * n) * m;
   float s[RMAX];
@@ -103,7 +105,7 @@ extern "C" int gs_linear_attention_scan(const void* x, int dtype, int ld, int oq
                                         const float* cos_t, const float* sin_t, int rd, int max_position,
                                         float key_scale, const float* decay, float* state, const int* q_start,
                                         const int* slots, const int* positions, float* out, int nseq, int H, int n,
-                                        int m, hipStream_t stream) {
+                                        int m, int below, hipStream_t stream) {
   GS_REQUIRE(nseq >= 0 && H > 0 && n > 0 && m > 0, "linear_attention: bad sizes nseq=%d H=%d n=%d m=%d", nseq, H, n, m);
   GS_REQUIRE(n <= 256, "linear_attention: keys of %d features, the kernel holds up to 256", n);
   GS_REQUIRE(H <= 65535 && (m + LA_COLS - 1) / LA_COLS <= 65535, "linear_attention: too many heads or value columns");
@@ -117,7 +119,7 @@ extern "C" int gs_linear_attention_scan(const void* x, int dtype, int ld, int oq
 #define LA_RUN(TI, R)                                                                                                \
   linear_attention_scan_kernel<TI, R><<<grid, 256, 0, stream>>>((const TI*)x, ld, oq, ok, ov, act, cos_t, sin_t, rd, \
                                                                 key_scale, decay, state, q_start, slots, positions,  \
-                                                                out, H, n, m)
+                                                                out, H, n, m, below)
 #define LA_RUN_T(TI)                      \
   if (n <= 32) LA_RUN(TI, 8);             \
   else if (n <= 64) LA_RUN(TI, 16);       \

@@ -1,0 +1,265 @@
+// Linear attention through a fading matrix state for prompt portions, on the matrix cores.
+//
+// The same recurrence as linear_attention.hip (S <- decay S + k_t v_t^T, o_t = S^T q_t, per sequence and head), taken
+// 32 tokens at a time.  With Q, K (32 x n) and V (32 x m) the rows of a run of L <= 32 tokens and S the state before it:
+//
+//   O  = diag(d^(t+1)) Q S  +  ((Q K^T) o D) V,     D[t][s] = d^(t-s) for s <= t, else 0
+//   S' = d^L S + sum_s d^(L-1-s) k_s v_s^T
+//
+// One block per (sequence, head, 128 value columns), four wavefronts, each owning 32 of the columns: its slice of the
+// state (transposed, 32 x n) stays in its accumulators from run to run.  Products are v_mfma_f32_32x32x16_bf16 with
+// float32 sums.  What the design holds in 32 bits (activated and turned q and k, the decayed scores, the state, the
+// decayed keys) enters the products as two bfloat16 terms, the value's rounding and the rounding of what is left, and
+// each product is three (hi hi + hi lo + lo hi): sixteen bits of every operand, the sums in float32.  Values enter as
+// one term (a projection with its activation).  Powers of the decay come from a table made by repeated multiplication.
+//
+// The scores are computed transposed (rows s, columns t), which leaves them, in a lane's registers, in the order in
+// which the next product takes its first operand, but for a permutation of the 16 inner indices of a step: slot q of
+// lane half hf stands for s = 16 step + 8 (q / 4) + 4 hf + q % 4; the value operand is read in the same order (two
+// 8-byte reads).  No trip of the scores through LDS, no wait between the two products.
+//
+// Sequences shorter than `min_len` tokens are left alone (the token-by-token kernel takes them).
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 lm_bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 lm_bf16x4_t;
+typedef __attribute__((ext_vector_type(16))) float lm_f32x16_t;
+
+constexpr int LM_C = 32;          // tokens a run
+constexpr int LM_MTB = 128;       // value columns a block
+constexpr int LM_LDT = LM_C + 8;  // elements per LDS row of the transposed operands
+
+__device__ __forceinline__ float lm_act(float z, int act) { return act ? z / (1.0f + expf(-z)) : z; }
+
+__device__ __forceinline__ void lm_split(float v, uint16_t& hi, uint16_t& lo) {
+  const bf16 h = f32_to_bf16(v);
+  hi = h.x;
+  lo = f32_to_bf16(v - to_f32(h)).x;
+}
+
+template <int NT>
+__global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
+    const bf16* __restrict__ x, int ld, int oq, int ok, int ov, int act, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int rd, float key_scale, const float* __restrict__ decay,
+    float* __restrict__ state, const int* __restrict__ q_start, const int* __restrict__ slots,
+    const int* __restrict__ positions, float* __restrict__ out, int H, int n, int m, int min_len) {
+  constexpr int NP = 32 * NT, LDQ = NP + 8;
+  extern __shared__ __align__(16) uint16_t lm_lds[];
+  uint16_t* Qh = lm_lds;  // [32][LDQ] each
+  uint16_t* Ql = Qh + LM_C * LDQ;
+  uint16_t* Kh = Ql + LM_C * LDQ;
+  uint16_t* Kl = Kh + LM_C * LDQ;
+  uint16_t* KTh = Kl + LM_C * LDQ;  // [NP][LDT] each: decayed keys, transposed
+  uint16_t* KTl = KTh + NP * LM_LDT;
+  uint16_t* VT = KTl + NP * LM_LDT;      // [MTB][LDT]: values, transposed
+  uint16_t* STh = VT + LM_MTB * LM_LDT;  // [MTB][LDQ] each: the state, transposed
+  uint16_t* STl = STh + LM_MTB * LDQ;
+  __shared__ float pw[LM_C + 1];
+
+  const int seq = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * LM_MTB;
+  const int t0 = q_start[seq], t1 = q_start[seq + 1];
+  if (t1 - t0 < min_len || t1 <= t0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+  const int jw = wave * 32;
+  const bool live = j0 + jw < m;      // a wavefront whose columns all lie beyond m only helps staging
+  const float d = decay[h];
+  float* S = state + (((size_t)slots[seq] * H + h) * n) * m;
+  if (tid == 0) {
+    float p = 1.f;
+    for (int e = 0; e <= LM_C; ++e) {
+      pw[e] = p;
+      p *= d;
+    }
+  }
+  lm_f32x16_t acc_s[NT];
+#pragma unroll
+  for (int it = 0; it < NT; ++it)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int i = it * 32 + l32, j = j0 + jw + 8 * (e / 4) + 4 * half + e % 4;
+      acc_s[it][e] = (i < n && j < m) ? S[(size_t)i * m + j] : 0.f;
+    }
+  const int hr = rd >> 1;
+
+  for (int tb = t0; tb < t1; tb += LM_C) {
+    const int nb = t1 - tb < LM_C ? t1 - tb : LM_C;
+    __syncthreads();  // the run before has been read (and, the first time, the table of powers is there)
+    for (int idx = tid; idx < LM_C * NP; idx += 256) {
+      const int t = idx / NP, i = idx - t * NP;
+      float qv = 0.f, kv = 0.f;
+      if (t < nb && i < n) {
+        const bf16* row = x + (size_t)(tb + t) * ld;
+        qv = lm_act(to_f32(row[oq + h * n + i]), act);
+        kv = lm_act(to_f32(row[ok + h * n + i]), act);
+        if (i < rd) {
+          const bool low = i < hr;
+          const int p = low ? i : i - hr, other = low ? i + hr : i - hr;
+          const size_t at = (size_t)positions[tb + t] * hr + p;
+          const float c = cos_t[at], sn = sin_t[at];
+          const float qo = lm_act(to_f32(row[oq + h * n + other]), act);
+          const float ko = lm_act(to_f32(row[ok + h * n + other]), act);
+          qv = low ? qv * c - qo * sn : qv * c + qo * sn;
+          kv = low ? kv * c - ko * sn : kv * c + ko * sn;
+        }
+        kv *= key_scale;
+      }
+      lm_split(qv, Qh[t * LDQ + i], Ql[t * LDQ + i]);
+      lm_split(kv, Kh[t * LDQ + i], Kl[t * LDQ + i]);
+      const float kd = t < nb ? kv * pw[nb - 1 - t] : 0.f;
+      lm_split(kd, KTh[i * LM_LDT + t], KTl[i * LM_LDT + t]);
+    }
+    for (int idx = tid; idx < LM_C * LM_MTB; idx += 256) {
+      const int t = idx / LM_MTB, c = idx - t * LM_MTB;
+      const int j = j0 + c;
+      const float v = (t < nb && j < m) ? lm_act(to_f32(x[(size_t)(tb + t) * ld + ov + h * m + j]), act) : 0.f;
+      VT[c * LM_LDT + t] = f32_to_bf16(v).x;
+    }
+    if (live) {
+#pragma unroll
+      for (int it = 0; it < NT; ++it)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int jj = jw + 8 * (e / 4) + 4 * half + e % 4, ii = it * 32 + l32;
+          lm_split(acc_s[it][e], STh[jj * LDQ + ii], STl[jj * LDQ + ii]);
+        }
+    }
+    __syncthreads();
+    if (!live) continue;
+
+    // scores, transposed: rows s, columns t
+    lm_f32x16_t at;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) at[e] = 0.f;
+    const int ro = l32 * LDQ + half * 8;
+#pragma unroll
+    for (int ks = 0; ks < NP / 16; ++ks) {
+      const lm_bf16x8_t kh8 = *reinterpret_cast<const lm_bf16x8_t*>(Kh + ro + ks * 16);
+      const lm_bf16x8_t kl8 = *reinterpret_cast<const lm_bf16x8_t*>(Kl + ro + ks * 16);
+      const lm_bf16x8_t qh8 = *reinterpret_cast<const lm_bf16x8_t*>(Qh + ro + ks * 16);
+      const lm_bf16x8_t ql8 = *reinterpret_cast<const lm_bf16x8_t*>(Ql + ro + ks * 16);
+      at = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh8, qh8, at, 0, 0, 0);
+      at = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh8, ql8, at, 0, 0, 0);
+      at = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kl8, qh8, at, 0, 0, 0);
+    }
+    // this lane: query t = l32, keys s(e); the causal rule and the decay between the two; as operands of the next product
+    lm_bf16x8_t ah[2], al[2];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int s = 8 * (e / 4) + 4 * half + e % 4;
+      const float a = s <= l32 ? at[e] * pw[l32 - s] : 0.f;
+      const bf16 hi = f32_to_bf16(a);
+      ah[e / 8][e % 8] = __builtin_bit_cast(__bf16, hi.x);
+      al[e / 8][e % 8] = __builtin_bit_cast(__bf16, f32_to_bf16(a - to_f32(hi)).x);
+    }
+    // what the state before the run gives: rows t, columns j, then each row times d^(t+1)
+    lm_f32x16_t o;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[e] = 0.f;
+    const int so = (jw + l32) * LDQ + half * 8;
+#pragma unroll
+    for (int ks = 0; ks < NP / 16; ++ks) {
+      const lm_bf16x8_t qh8 = *reinterpret_cast<const lm_bf16x8_t*>(Qh + ro + ks * 16);
+      const lm_bf16x8_t ql8 = *reinterpret_cast<const lm_bf16x8_t*>(Ql + ro + ks * 16);
+      const lm_bf16x8_t sh8 = *reinterpret_cast<const lm_bf16x8_t*>(STh + so + ks * 16);
+      const lm_bf16x8_t sl8 = *reinterpret_cast<const lm_bf16x8_t*>(STl + so + ks * 16);
+      o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qh8, sh8, o, 0, 0, 0);
+      o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qh8, sl8, o, 0, 0, 0);
+      o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ql8, sh8, o, 0, 0, 0);
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[e] *= pw[8 * (e / 4) + 4 * half + e % 4 + 1];
+    // what the run's own tokens give
+    const int vo = (jw + l32) * LM_LDT;
+#pragma unroll
+    for (int k2 = 0; k2 < 2; ++k2) {
+      const lm_bf16x4_t v0 = *reinterpret_cast<const lm_bf16x4_t*>(VT + vo + 16 * k2 + 4 * half);
+      const lm_bf16x4_t v1 = *reinterpret_cast<const lm_bf16x4_t*>(VT + vo + 16 * k2 + 8 + 4 * half);
+      lm_bf16x8_t v8;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        v8[q] = v0[q];
+        v8[4 + q] = v1[q];
+      }
+      o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[k2], v8, o, 0, 0, 0);
+      o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[k2], v8, o, 0, 0, 0);
+    }
+    {
+      const int j = j0 + jw + l32;
+      if (j < m) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int t = 8 * (e / 4) + 4 * half + e % 4;
+          if (t < nb) out[((size_t)(tb + t) * H + h) * m + j] = o[e];
+        }
+      }
+    }
+    // the state after the run: rows j, columns i
+    const float dl = pw[nb];
+#pragma unroll
+    for (int it = 0; it < NT; ++it) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc_s[it][e] *= dl;
+#pragma unroll
+      for (int k2 = 0; k2 < 2; ++k2) {
+        const lm_bf16x8_t v8 = *reinterpret_cast<const lm_bf16x8_t*>(VT + vo + 16 * k2 + 8 * half);
+        const int ko = (it * 32 + l32) * LM_LDT + 16 * k2 + 8 * half;
+        const lm_bf16x8_t kh8 = *reinterpret_cast<const lm_bf16x8_t*>(KTh + ko);
+        const lm_bf16x8_t kl8 = *reinterpret_cast<const lm_bf16x8_t*>(KTl + ko);
+        acc_s[it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v8, kh8, acc_s[it], 0, 0, 0);
+        acc_s[it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v8, kl8, acc_s[it], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NT; ++it)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int i = it * 32 + l32, j = j0 + jw + 8 * (e / 4) + 4 * half + e % 4;
+      if (i < n && j < m) S[(size_t)i * m + j] = acc_s[it][e];
+    }
+}
+
+template <int NT>
+static void lm_launch(dim3 grid, hipStream_t stream, const bf16* x, int ld, int oq, int ok, int ov, int act,
+                      const float* cos_t, const float* sin_t, int rd, float key_scale, const float* decay, float* state,
+                      const int* q_start, const int* slots, const int* positions, float* out, int H, int n, int m,
+                      int min_len) {
+  constexpr int NP = 32 * NT, LDQ = NP + 8;
+  const size_t lds = (size_t)(4 * LM_C * LDQ + 2 * NP * LM_LDT + LM_MTB * LM_LDT + 2 * LM_MTB * LDQ) * sizeof(uint16_t);
+  // more than the default limit of dynamic LDS: asked for once per kernel
+  static const hipError_t asked = hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_attention_chunk_kernel<NT>),
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  (void)asked;
+  linear_attention_chunk_kernel<NT><<<grid, 256, lds, stream>>>(x, ld, oq, ok, ov, act, cos_t, sin_t, rd, key_scale,
+                                                                decay, state, q_start, slots, positions, out, H, n, m,
+                                                                min_len);
+}
+
+extern "C" int gs_linear_attention_chunks_max_key() { return 128; }
+
+extern "C" int gs_linear_attention_chunks(const void* x, int ld, int oq, int ok, int ov, int act, const float* cos_t,
+                                          const float* sin_t, int rd, int max_position, float key_scale,
+                                          const float* decay, float* state, const int* q_start, const int* slots,
+                                          const int* positions, float* out, int nseq, int H, int n, int m, int min_len,
+                                          hipStream_t stream) {
+  GS_REQUIRE(nseq >= 0 && H > 0 && n > 0 && m > 0, "linear_attention_chunks: bad sizes nseq=%d H=%d n=%d m=%d", nseq, H, n, m);
+  GS_REQUIRE(n <= 128, "linear_attention_chunks: keys of %d features, the kernel holds up to 128", n);
+  GS_REQUIRE(H <= 65535 && (m + LM_MTB - 1) / LM_MTB <= 65535, "linear_attention_chunks: too many heads or value columns");
+  GS_REQUIRE(rd >= 0 && rd <= n && rd % 2 == 0, "linear_attention_chunks: %d turned features of %d", rd, n);
+  GS_REQUIRE(rd == 0 || (cos_t && sin_t && max_position > 0), "linear_attention_chunks: rotation without a table");
+  GS_REQUIRE(oq >= 0 && ok >= 0 && ov >= 0 && oq + H * n <= ld && ok + H * n <= ld && ov + H * m <= ld,
+             "linear_attention_chunks: q, k or v lie outside the rows of %d", ld);
+  GS_REQUIRE(act == 0 || act == 1, "linear_attention_chunks: unknown activation %d", act);
+  if (nseq == 0) return 0;
+  dim3 grid(nseq, H, (m + LM_MTB - 1) / LM_MTB);
+#define LM_RUN(NT)                                                                                                   \
+  lm_launch<NT>(grid, stream, (const bf16*)x, ld, oq, ok, ov, act, cos_t, sin_t, rd, key_scale, decay, state, q_start, \
+                slots, positions, out, H, n, m, min_len)
+  if (n <= 32) LM_RUN(1);
+  else if (n <= 64) LM_RUN(2);
+  else if (n <= 96) LM_RUN(3);
+  else LM_RUN(4);
+#undef LM_RUN
+  GS_LAUNCH_CHECK("linear_attention_chunks");
+  return 0;
+}

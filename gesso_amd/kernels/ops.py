@@ -385,17 +385,22 @@ _ACTS = {None: 0, "none": 0, "silu": 1}
 _GATES = {"sigmoid": 0, "silu": 1}
 GATED_ACTS = {"silu": 0, "gelu_tanh": 1}
 LINEAR_ATTENTION_MAX_KEY = 256
+LINEAR_ATTENTION_CHUNKS_MAX_KEY = 128
 
 
 def linear_attention_scan(x, oq: int, ok: int, ov: int, H: int, n: int, m: int, decay, state, q_start, slots, positions,
                           nseq: int, activation=None, cos=None, sin=None, rotary_dim: int = 0, key_scale: float = 1.0,
-                          out: torch.Tensor = None) -> torch.Tensor:
+                          out: torch.Tensor = None, below: int = 0, chunks_from: int = 0) -> torch.Tensor:
     """Linear attention through a fading state: per sequence and head ``S <- decay_h S + k_t v_t^T``, ``o_t = S^T q_t``.
 
     ``x (T, ld)`` holds q of head h at columns ``[oq + h n, ...)``, k at ``[ok + h n, ...)``, v at ``[ov + h m, ...)``;
     ``activation`` (None or ``"silu"``) is applied to all three, q and k are turned by ``positions`` over their first
     ``rotary_dim`` features (half-split pairs, tables ``(P, rotary_dim/2)``), k is multiplied by ``key_scale``.
-    ``state (slots, H, n, m)`` float32 is read and advanced for the sequences' ``slots``.  Returns ``(T, H m)`` float32."""
+    ``state (slots, H, n, m)`` float32 is read and advanced for the sequences' ``slots``.  Returns ``(T, H m)`` float32.
+
+    ``below`` > 0: only the sequences that bring fewer tokens than that (the rows of the others are left as they are).
+    ``chunks_from`` > 0: the kernel on the matrix cores instead (bfloat16 rows, keys up to
+    ``LINEAR_ATTENTION_CHUNKS_MAX_KEY`` wide), for the sequences that bring at least that many tokens."""
     _dev(x, decay, state, q_start, slots, positions, cos, sin, out)
     _need(x.dim() == 2, "linear_attention: rows (T, ld)")
     T, ld = x.shape
@@ -415,11 +420,20 @@ def linear_attention_scan(x, oq: int, ok: int, ov: int, H: int, n: int, m: int, 
     if out is None:
         out = torch.empty((T, H * m), dtype=torch.float32, device=x.device)
     _need(out.shape == (T, H * m) and out.dtype == torch.float32, "linear_attention: out must be float32 (T, H m)")
+    if chunks_from > 0:
+        _need(x.dtype == torch.bfloat16 and n <= LINEAR_ATTENTION_CHUNKS_MAX_KEY,
+              "linear_attention: the kernel on the matrix cores takes bfloat16 rows and keys up to 128 wide")
+        _check(lib().gs_linear_attention_chunks(_p(x), c_int(ld), c_int(oq), c_int(ok), c_int(ov), c_int(_ACTS[activation]),
+                                                _p(cos) if rotary_dim else None, _p(sin) if rotary_dim else None,
+                                                c_int(rotary_dim), c_int(max_pos), c_float(key_scale), _p(decay), _p(state),
+                                                _p(q_start), _p(slots), _p(positions), _p(out), c_int(nseq), c_int(H),
+                                                c_int(n), c_int(m), c_int(chunks_from), _stream()))
+        return out
     _check(lib().gs_linear_attention_scan(_p(x), c_int(_dt(x)), c_int(ld), c_int(oq), c_int(ok), c_int(ov),
                                           c_int(_ACTS[activation]), _p(cos) if rotary_dim else None,
                                           _p(sin) if rotary_dim else None, c_int(rotary_dim), c_int(max_pos),
                                           c_float(key_scale), _p(decay), _p(state), _p(q_start), _p(slots), _p(positions),
-                                          _p(out), c_int(nseq), c_int(H), c_int(n), c_int(m), _stream()))
+                                          _p(out), c_int(nseq), c_int(H), c_int(n), c_int(m), c_int(below), _stream()))
     return out
 
 

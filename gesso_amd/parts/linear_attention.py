@@ -23,6 +23,7 @@ from .registry import build, part_class, register
 class LinearAttention(Part):
     graph_safe = True
     stage, out_stage = "linear_mixer", "linear_out"
+    RUNS_FROM = 8       # sequences that bring at least this many tokens to a step go to the kernel on the matrix cores
 
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
@@ -68,9 +69,18 @@ class LinearAttention(Part):
         with rt.stage("linear_in"):
             rows = rt.linear(rt.dense(x), self.w_in)                   # q | k | v | g
         with rt.stage("linear_state"):
-            o = ops.linear_attention_scan(rows, 0, H * n, 2 * H * n, H, n, m, self.decay, cache.state["state"],
-                                          ctx.q_start, ctx.slots, ctx.positions, ctx.nseq, activation=s.activation,
-                                          cos=pos.cos, sin=pos.sin, rotary_dim=pos.rotary_dim, key_scale=s.key_scale)
+            args = (rows, 0, H * n, 2 * H * n, H, n, m, self.decay, cache.state["state"], ctx.q_start, ctx.slots,
+                    ctx.positions, ctx.nseq)
+            kw = dict(activation=s.activation, cos=pos.cos, sin=pos.sin, rotary_dim=pos.rotary_dim, key_scale=s.key_scale)
+            runs = (rt.options.linear_attention == "auto" and rows.dtype == torch.bfloat16 and not ctx.all_single
+                    and n <= ops.LINEAR_ATTENTION_CHUNKS_MAX_KEY and ctx.max_q_len >= self.RUNS_FROM)
+            if runs:
+                # prompt portions 32 tokens at a time on the matrix cores; what brings fewer tokens, token by token
+                o = ops.linear_attention_scan(*args, chunks_from=self.RUNS_FROM, **kw)
+                if min(ctx.q_lens) < self.RUNS_FROM:
+                    ops.linear_attention_scan(*args, below=self.RUNS_FROM, out=o, **kw)
+            else:
+                o = ops.linear_attention_scan(*args, **kw)
         with rt.stage("linear_norm"):
             return ops.gated_outnorm(o, rows, 2 * H * n + H * m, self.norm_weight, s.eps, H, m, s.out_norm == "joint",
                                      s.gate, rt.dtype)

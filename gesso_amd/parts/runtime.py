@@ -45,6 +45,9 @@ class RuntimeOptions:
     takes the sizes, ``"general"`` = the general float32-arithmetic kernel always.
     ``routed_experts``: a table-routed mixture of experts in bfloat16: ``"auto"`` = pairs sorted by expert and products on
     the matrix cores once a step's (token, choice) pairs outnumber the experts twice over, ``"token"`` = token by token always.
+    ``linear_attention``: linear attention through a fading state in bfloat16: ``"auto"`` = prompt portions 32 tokens at a
+    time on the matrix cores (operands that the design holds in 32 bits as two bfloat16 terms), ``"token"`` = token by
+    token in float32 arithmetic always.
     ``tiled_rows``: rows handed from one fused kernel to the next product travel in the order the matrix cores
     take them (``ops.TiledRows``): a product then loads them a contiguous kilobyte at a time.
     ``tile_weights``: keep a tile-major copy of each bfloat16 weight for the streaming kernels.
@@ -65,6 +68,7 @@ class RuntimeOptions:
     prompt_attention: str = "auto"
     latent_attention: str = "auto"
     routed_experts: str = "auto"
+    linear_attention: str = "auto"
     tiled_rows: bool = True
     tile_weights: bool = True
     fold_norm_rows: int = 0
@@ -79,6 +83,8 @@ class RuntimeOptions:
             raise KernelError(f"latent_attention is 'auto' or 'general', not {self.latent_attention!r}")
         if self.routed_experts not in ("auto", "token"):
             raise KernelError(f"routed_experts is 'auto' or 'token', not {self.routed_experts!r}")
+        if self.linear_attention not in ("auto", "token"):
+            raise KernelError(f"linear_attention is 'auto' or 'token', not {self.linear_attention!r}")
         if self.fold_norm_rows < 0 or self.weighted_rows_max < 0:
             raise KernelError("row limits are nonnegative")
 

@@ -90,7 +90,8 @@ def test_weighted_sum_of_two_results(ops):
     assert torch.allclose(ops.scaled_sum(a.to(DEV), 0.3, b.to(DEV), 2.0, torch.float32).cpu(), 0.3 * a + 2.0 * b, atol=1e-6)
 
 
-def scan_case(ops, dtype, H, n, m, lens, rd=0, act=None, scale=1.0, decay=None, seed=0, base=1e3, pos0=None, boost=None):
+def scan_case(ops, dtype, H, n, m, lens, rd=0, act=None, scale=1.0, decay=None, seed=0, base=1e3, pos0=None, boost=None,
+              runs_from=0):
     """Rows of q | junk | k | v for sequences of ``lens`` tokens, states in shuffled slots: the kernel's outputs and
     states, and the plain implementation's.  ``pos0``: the first position of each sequence (its state then starts from
     a random one).  ``boost``: ``(sequence, far token, near token)``: that key and that query are made to meet."""
@@ -123,9 +124,16 @@ def scan_case(ops, dtype, H, n, m, lens, rd=0, act=None, scale=1.0, decay=None, 
         ang = torch.arange(max(positions) + 1, dtype=torch.float64)[:, None] * torch.tensor(f, dtype=torch.float64)[None]
         cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
     st = state.to(DEV)
-    out = ops.linear_attention_scan(x.to(DEV), 0, H * n + junk, 2 * H * n + junk, H, n, m,
-                                    torch.tensor(decay, dtype=torch.float32, device=DEV), st, i32(q_start), i32(slots),
-                                    i32(positions), len(lens), activation=act, cos=cos, sin=sin, rotary_dim=rd, key_scale=scale)
+    args = (x.to(DEV), 0, H * n + junk, 2 * H * n + junk, H, n, m, torch.tensor(decay, dtype=torch.float32, device=DEV), st,
+            i32(q_start), i32(slots), i32(positions), len(lens))
+    kw = dict(activation=act, cos=cos, sin=sin, rotary_dim=rd, key_scale=scale)
+    if runs_from:
+        # sequences of at least that many tokens on the matrix cores, the others token by token, into one result
+        out = torch.full((T, H * m), float("nan"), device=DEV)
+        ops.linear_attention_scan(*args, chunks_from=runs_from, out=out, **kw)
+        ops.linear_attention_scan(*args, below=runs_from, out=out, **kw)
+    else:
+        out = ops.linear_attention_scan(*args, **kw)
     xd = x.double()
     fa = P.silu if act == "silu" else (lambda z: z)
     want, want_state = [], {}
@@ -157,6 +165,25 @@ def test_fading_state_kernel_over_unequal_sequences(ops, dtype, H, n, m, rd, act
     assert float((got - want).abs().max()) <= 5e-5 * max(1.0, float(want.abs().max()))     # float32 arithmetic in both types
     for slot, S in want_state.items():
         assert float((state[slot] - S).abs().max()) <= 5e-5 * max(1.0, float(S.abs().max()))
+    untouched = [s for s in range(state.shape[0]) if s not in want_state]
+    assert all(torch.isnan(state[s]).all() for s in untouched)
+
+
+@pytest.mark.parametrize("H,n,m,rd,act,scale,decay", [
+    (3, 24, 16, 0, "silu", 1.0, None), (2, 16, 24, 8, None, 0.25, None), (1, 40, 48, 40, None, 0.5, None),
+    (2, 64, 64, 0, "silu", 1.0, (0.97, 0.999)), (1, 128, 130, 64, None, 0.1, (0.99,)), (5, 6, 10, 2, None, 1.0, (0.0, 0.5, 0.9, 1.0, 0.999)),
+    (2, 128, 128, 0, "silu", 1.0, (1.0, 0.9)), (2, 32, 64, 32, None, 32 ** -0.5, None), (1, 96, 300, 10, None, 0.2, None)])
+def test_fading_state_kernel_on_the_matrix_cores(ops, H, n, m, rd, act, scale, decay):
+    """Prompt portions 32 tokens at a time: whole runs, a last run of one token, sequences below the kernel's least
+    length beside it, states that go on from earlier steps (positions deep in a sequence)."""
+    lens, pos0 = [1, 70, 9, 33, 8, 140, 32, 7], [5, 0, 100, 0, 31, 12, 0, 0]
+    got, want, state, want_state = scan_case(ops, torch.bfloat16, H, n, m, lens, rd, act, scale, decay=decay and list(decay),
+                                             seed=n + m, pos0=pos0, runs_from=8)
+    # activated values enter the products as one bfloat16 term (a projection with its activation); all else as two
+    bound = 4e-3 if act else 1e-4
+    assert float((got - want).abs().max()) <= bound * max(1.0, float(want.abs().max()))
+    for slot, S in want_state.items():
+        assert float((state[slot] - S).abs().max()) <= bound * max(1.0, float(S.abs().max()))
     untouched = [s for s in range(state.shape[0]) if s not in want_state]
     assert all(torch.isnan(state[s]).all() for s in untouched)
 
