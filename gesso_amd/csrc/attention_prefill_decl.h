@@ -6,6 +6,7 @@ struct PrefillCall {
   const bf16 *q, *kc, *vc;
   const int *positions, *tile_seq, *tile_row, *tile_n, *bt;
   int q_stride, max_blocks, page_size, window, nh, nkv, tile_rows, ntiles;
+  int chunk, sink;
   unsigned page_magic;
   float scale;
   bf16* out;

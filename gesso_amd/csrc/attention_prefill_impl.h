@@ -14,7 +14,9 @@
 // No probability ever crosses lanes; the only cross-lane traffic is the maximum and the sum over the four
 // lane groups.  v_mfma_f32_16x16x32_bf16 throughout.
 //
-// Causal rule: the query at position p sees keys lo..p, lo = 0 or p - window + 1.  Tiles of queries come
+// Causal rule: the query at position p sees keys lo..p, lo = 0 or p - window + 1; with chunk > 0 no further back
+// than the first position of p's own run of `chunk` positions.  With `sink` the softmax's denominator has one more
+// term, exp(0), which has no value.  Tiles of queries come
 // from the host: tile i covers rows tile_row[i] .. + tile_n[i] (at most 16 QT) of the flattened tokens, of
 // sequence tile_seq[i].  Exponentials are base 2 on scores scaled by log2(e): one v_exp_f32 each.  q (T, q_stride), head h at [h D, (h+1) D); caches (pages, nkv, page_size, D); out (T, nh D).
 #pragma once
@@ -39,7 +41,7 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
     const int* __restrict__ positions, const int* __restrict__ tile_seq, const int* __restrict__ tile_row,
     const int* __restrict__ tile_n, const int* __restrict__ block_table, int max_blocks, int page_size,
-    unsigned page_magic, int window, float scale, bf16* __restrict__ out, int nh, int nkv) {
+    unsigned page_magic, int window, float scale, bf16* __restrict__ out, int nh, int nkv, int chunk, int sink) {
   constexpr int PF_KSTEP = D <= 64 ? 64 : 32;   // keys per step: what three sets of row registers allow
   constexpr int KK = D / 32;   // feature steps of the score product
   constexpr int DT = D / 16;   // feature tiles of the output
@@ -59,7 +61,14 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
   const int* bt = block_table + (size_t)seq * max_blocks;
   const int pos0 = positions[row0];                  // positions of a tile are consecutive
   const int last_key = pos0 + nq - 1;
-  const int first_key = window > 0 ? (pos0 - window + 1 > 0 ? pos0 - window + 1 : 0) : 0;
+  // the first key that the query at position p sees: a window's, and with chunk > 0 the first of p's own run of
+  // `chunk` positions (runs are counted from position 0); it never falls as p grows
+  auto lo_of = [&](int p) -> int {
+    int lo = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+    if (chunk > 0 && p - p % chunk > lo) lo = p - p % chunk;
+    return lo;
+  };
+  const int first_key = lo_of(pos0);
   // scores are kept in units of log2(e), so that the exponentials are single v_exp_f32
   const float sc = scale * PF_LOG2E;
 
@@ -71,7 +80,7 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
     const int r = t * 16 + r16;
     live[t] = r < nq;
     my_pos[t] = pos0 + (live[t] ? r : nq - 1);
-    my_lo[t] = window > 0 ? (my_pos[t] - window + 1 > 0 ? my_pos[t] - window + 1 : 0) : 0;
+    my_lo[t] = lo_of(my_pos[t]);
     const bf16* qrow = q + (size_t)(row0 + (live[t] ? r : 0)) * q_stride + (size_t)h * D + kg * 8;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) qf[t][kk] = *reinterpret_cast<const bf16x8_t*>(qrow + kk * 32);
@@ -224,7 +233,7 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
         for (int t = 0; t < QT; ++t) acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pf[t][ns], acc[t][dt], 0, 0, 0);
       }
   };
-  const int last_lo = window > 0 ? (last_key - window + 1 > 0 ? last_key - window + 1 : 0) : 0;
+  const int last_lo = lo_of(last_key);
   auto step = [&](auto stage, int k0) {
     const bool inner = k0 + PF_KSTEP - 1 <= pos0 && k0 >= last_lo && k0 >= win_first && k0 + PF_KSTEP - 1 <= win_last &&
                        nq == 16 * QT;
@@ -294,6 +303,8 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
     if (!live[t]) continue;
+    // a sink: one more term in the denominator, of score 0 (scores are held relative to m, in units of log2 e)
+    if (sink) l[t] += m[t] == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(-m[t]);
     const float inv = 1.0f / l[t];
     bf16* orow = out + (size_t)(row0 + t * 16 + r16) * nh * D + (size_t)h * D;
 #pragma unroll
@@ -310,12 +321,12 @@ template <int D, int QT, int KSPLIT>
 static int launch_prefill(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, const bf16* kc,
                           const bf16* vc, const int* positions, const int* tile_seq, const int* tile_row,
                           const int* tile_n, const int* bt, int max_blocks, int page_size, unsigned page_magic,
-                          int window, float scale, bf16* out, int nh, int nkv) {
+                          int window, float scale, bf16* out, int nh, int nkv, int chunk, int sink) {
 #define GS_RUN(GG)                                                                                                   \
   if constexpr (KSPLIT > 1 && GG > 4) return -1;                                                                        \
   else attention_prefill_kernel<D, GG, QT, KSPLIT><<<grid, GG * KSPLIT * 64, 0, stream>>>(q, q_stride, kc, vc, positions, tile_seq, tile_row, \
                                                                 tile_n, bt, max_blocks, page_size, page_magic, window, \
-                                                                scale, out, nh, nkv)
+                                                                scale, out, nh, nkv, chunk, sink)
   switch (G) {
     case 1: GS_RUN(1); break;
     case 2: GS_RUN(2); break;
@@ -342,7 +353,7 @@ static int prefill_for_width(const PrefillCall& c) {
   const bool split = G <= 4;
 #define GS_ARGS                                                                                                    \
   G, grid, c.stream, c.q, c.q_stride, c.kc, c.vc, c.positions, c.tile_seq, c.tile_row, c.tile_n, c.bt, c.max_blocks, \
-      c.page_size, c.page_magic, c.window, c.scale, c.out, c.nh, c.nkv
+      c.page_size, c.page_magic, c.window, c.scale, c.out, c.nh, c.nkv, c.chunk, c.sink
   if (c.tile_rows == 16) return split ? launch_prefill<D, 1, 2>(GS_ARGS) : launch_prefill<D, 1, 1>(GS_ARGS);
   return split ? launch_prefill<D, 2, 2>(GS_ARGS) : launch_prefill<D, 2, 1>(GS_ARGS);
 #undef GS_ARGS

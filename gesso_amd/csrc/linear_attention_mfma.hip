@@ -29,7 +29,10 @@ constexpr int LM_C = 32;          // tokens a run
 constexpr int LM_MTB = 128;       // value columns a block
 constexpr int LM_LDT = LM_C + 8;  // elements per LDS row of the transposed operands
 
-__device__ __forceinline__ float lm_act(float z, int act) { return act ? z / (1.0f + expf(-z)) : z; }
+// silu by the hardware's exponential and reciprocal (each good to a unit in the last place of float32)
+__device__ __forceinline__ float lm_act(float z, int act) {
+  return act ? z * __builtin_amdgcn_rcpf(1.0f + __expf(-z)) : z;
+}
 
 __device__ __forceinline__ void lm_split(float v, uint16_t& hi, uint16_t& lo) {
   const bf16 h = f32_to_bf16(v);
@@ -37,7 +40,7 @@ __device__ __forceinline__ void lm_split(float v, uint16_t& hi, uint16_t& lo) {
   lo = f32_to_bf16(v - to_f32(h)).x;
 }
 
-template <int NT>
+template <int NT, bool VEC>
 __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
     const bf16* __restrict__ x, int ld, int oq, int ok, int ov, int act, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int rd, float key_scale, const float* __restrict__ decay,
@@ -81,38 +84,133 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
     }
   const int hr = rd >> 1;
 
+  // VEC: a run's rows come as 16-byte pieces (eight features of one token), all of a thread's pieces asked for at once
+  // and, from the second run on, while the run before is still being computed.  Piece u of a thread: token
+  // (tid + 256 u) % 32, features 8 ((tid + 256 u) / 32) ... (neighbouring lanes hold neighbouring tokens, so that the
+  // transposed stores into LDS fall side by side); a piece's partner in the turn is a whole piece too (rd / 2 a
+  // multiple of eight).  Values: piece (tid + 256 u) % 32 -> token, / 32 -> eight columns.
+  constexpr int UQ = (LM_C * NP / 8 + 255) / 256, UV = LM_C * LM_MTB / 8 / 256;
+  uint4 rq[UQ], rk[UQ], rqo[UQ], rko[UQ], rv[UV];
+  const int pos0 = positions[t0];
+  auto fetch = [&](int tb, int nb) {
+    if constexpr (VEC) {
+#pragma unroll
+      for (int u = 0; u < UQ; ++u) {
+        const int piece = tid + 256 * u, t = piece % LM_C, i = (piece / LM_C) * 8;
+        rq[u] = rk[u] = rqo[u] = rko[u] = make_uint4(0, 0, 0, 0);
+        if (t < nb && i < n) {
+          const bf16* row = x + (size_t)(tb + t) * ld;
+          rq[u] = *reinterpret_cast<const uint4*>(row + oq + h * n + i);
+          rk[u] = *reinterpret_cast<const uint4*>(row + ok + h * n + i);
+          if (i < rd) {
+            const int other = i < hr ? i + hr : i - hr;
+            rqo[u] = *reinterpret_cast<const uint4*>(row + oq + h * n + other);
+            rko[u] = *reinterpret_cast<const uint4*>(row + ok + h * n + other);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UV; ++u) {
+        const int piece = tid + 256 * u, t = piece % LM_C, c = (piece / LM_C) * 8;
+        rv[u] = make_uint4(0, 0, 0, 0);
+        if (t < nb && j0 + c < m) rv[u] = *reinterpret_cast<const uint4*>(x + (size_t)(tb + t) * ld + ov + h * m + j0 + c);
+      }
+    }
+  };
+  auto eight = [](const uint4& w, float* v) {
+    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[2 * e] = __uint_as_float(ww[e] << 16);
+      v[2 * e + 1] = __uint_as_float(ww[e] & 0xffff0000u);
+    }
+  };
+  if (t1 > t0) fetch(t0, t1 - t0 < LM_C ? t1 - t0 : LM_C);
+
   for (int tb = t0; tb < t1; tb += LM_C) {
     const int nb = t1 - tb < LM_C ? t1 - tb : LM_C;
     __syncthreads();  // the run before has been read (and, the first time, the table of powers is there)
-    for (int idx = tid; idx < LM_C * NP; idx += 256) {
-      const int t = idx / NP, i = idx - t * NP;
-      float qv = 0.f, kv = 0.f;
-      if (t < nb && i < n) {
-        const bf16* row = x + (size_t)(tb + t) * ld;
-        qv = lm_act(to_f32(row[oq + h * n + i]), act);
-        kv = lm_act(to_f32(row[ok + h * n + i]), act);
-        if (i < rd) {
-          const bool low = i < hr;
-          const int p = low ? i : i - hr, other = low ? i + hr : i - hr;
-          const size_t at = (size_t)positions[tb + t] * hr + p;
-          const float c = cos_t[at], sn = sin_t[at];
-          const float qo = lm_act(to_f32(row[oq + h * n + other]), act);
-          const float ko = lm_act(to_f32(row[ok + h * n + other]), act);
-          qv = low ? qv * c - qo * sn : qv * c + qo * sn;
-          kv = low ? kv * c - ko * sn : kv * c + ko * sn;
+    if constexpr (VEC) {
+#pragma unroll
+      for (int u = 0; u < UQ; ++u) {
+        const int piece = tid + 256 * u, t = piece % LM_C, i = (piece / LM_C) * 8;
+        if (i >= NP) continue;
+        float q8[8], k8[8], qo[8], ko[8];
+        eight(rq[u], q8);
+        eight(rk[u], k8);
+        eight(rqo[u], qo);
+        eight(rko[u], ko);
+        const bool turned = t < nb && i < rd, low = i < hr;
+        float c8[8], s8[8];
+        if (turned) {
+          const float* cr = cos_t + (size_t)(pos0 + tb - t0 + t) * hr + (low ? i : i - hr);
+          const float* sr = sin_t + (size_t)(pos0 + tb - t0 + t) * hr + (low ? i : i - hr);
+          load8f(cr, c8);
+          load8f(sr, s8);
         }
-        kv *= key_scale;
+        const float kdec = t < nb ? pw[nb - 1 - t] : 0.f;
+        uint16_t qh[8], ql[8], kh[8], kl[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float qv = lm_act(q8[e], act), kv = lm_act(k8[e], act);
+          if (turned) {
+            const float qp = lm_act(qo[e], act), kp = lm_act(ko[e], act);
+            qv = low ? qv * c8[e] - qp * s8[e] : qv * c8[e] + qp * s8[e];
+            kv = low ? kv * c8[e] - kp * s8[e] : kv * c8[e] + kp * s8[e];
+          }
+          kv *= key_scale;
+          lm_split(qv, qh[e], ql[e]);
+          lm_split(kv, kh[e], kl[e]);
+          lm_split(kv * kdec, KTh[(i + e) * LM_LDT + t], KTl[(i + e) * LM_LDT + t]);
+        }
+        auto pack = [](const uint16_t* v) {
+          return make_uint4(v[0] | ((uint32_t)v[1] << 16), v[2] | ((uint32_t)v[3] << 16), v[4] | ((uint32_t)v[5] << 16),
+                            v[6] | ((uint32_t)v[7] << 16));
+        };
+        *reinterpret_cast<uint4*>(Qh + t * LDQ + i) = pack(qh);
+        *reinterpret_cast<uint4*>(Ql + t * LDQ + i) = pack(ql);
+        *reinterpret_cast<uint4*>(Kh + t * LDQ + i) = pack(kh);
+        *reinterpret_cast<uint4*>(Kl + t * LDQ + i) = pack(kl);
       }
-      lm_split(qv, Qh[t * LDQ + i], Ql[t * LDQ + i]);
-      lm_split(kv, Kh[t * LDQ + i], Kl[t * LDQ + i]);
-      const float kd = t < nb ? kv * pw[nb - 1 - t] : 0.f;
-      lm_split(kd, KTh[i * LM_LDT + t], KTl[i * LM_LDT + t]);
-    }
-    for (int idx = tid; idx < LM_C * LM_MTB; idx += 256) {
-      const int t = idx / LM_MTB, c = idx - t * LM_MTB;
-      const int j = j0 + c;
-      const float v = (t < nb && j < m) ? lm_act(to_f32(x[(size_t)(tb + t) * ld + ov + h * m + j]), act) : 0.f;
-      VT[c * LM_LDT + t] = f32_to_bf16(v).x;
+#pragma unroll
+      for (int u = 0; u < UV; ++u) {
+        const int piece = tid + 256 * u, t = piece % LM_C, c = (piece / LM_C) * 8;
+        float v8[8];
+        eight(rv[u], v8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) VT[(c + e) * LM_LDT + t] = f32_to_bf16(lm_act(v8[e], act)).x;
+      }
+    } else {
+      for (int idx = tid; idx < LM_C * NP; idx += 256) {
+        const int t = idx / NP, i = idx - t * NP;
+        float qv = 0.f, kv = 0.f;
+        if (t < nb && i < n) {
+          const bf16* row = x + (size_t)(tb + t) * ld;
+          qv = lm_act(to_f32(row[oq + h * n + i]), act);
+          kv = lm_act(to_f32(row[ok + h * n + i]), act);
+          if (i < rd) {
+            const bool low = i < hr;
+            const int p = low ? i : i - hr, other = low ? i + hr : i - hr;
+            const size_t at = (size_t)positions[tb + t] * hr + p;
+            const float c = cos_t[at], sn = sin_t[at];
+            const float qo = lm_act(to_f32(row[oq + h * n + other]), act);
+            const float ko = lm_act(to_f32(row[ok + h * n + other]), act);
+            qv = low ? qv * c - qo * sn : qv * c + qo * sn;
+            kv = low ? kv * c - ko * sn : kv * c + ko * sn;
+          }
+          kv *= key_scale;
+        }
+        lm_split(qv, Qh[t * LDQ + i], Ql[t * LDQ + i]);
+        lm_split(kv, Kh[t * LDQ + i], Kl[t * LDQ + i]);
+        const float kd = t < nb ? kv * pw[nb - 1 - t] : 0.f;
+        lm_split(kd, KTh[i * LM_LDT + t], KTl[i * LM_LDT + t]);
+      }
+      for (int idx = tid; idx < LM_C * LM_MTB; idx += 256) {
+        const int t = idx / LM_MTB, c = idx - t * LM_MTB;
+        const int j = j0 + c;
+        const float v = (t < nb && j < m) ? lm_act(to_f32(x[(size_t)(tb + t) * ld + ov + h * m + j]), act) : 0.f;
+        VT[c * LM_LDT + t] = f32_to_bf16(v).x;
+      }
     }
     if (live) {
 #pragma unroll
@@ -124,6 +222,7 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
         }
     }
     __syncthreads();
+    if (tb + LM_C < t1) fetch(tb + LM_C, t1 - tb - LM_C < LM_C ? t1 - tb - LM_C : LM_C);   // the next run's rows, meanwhile
     if (!live) continue;
 
     // scores, transposed: rows s, columns t
@@ -219,7 +318,7 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
     }
 }
 
-template <int NT>
+template <int NT, bool VEC>
 static void lm_launch(dim3 grid, hipStream_t stream, const bf16* x, int ld, int oq, int ok, int ov, int act,
                       const float* cos_t, const float* sin_t, int rd, float key_scale, const float* decay, float* state,
                       const int* q_start, const int* slots, const int* positions, float* out, int H, int n, int m,
@@ -227,10 +326,10 @@ static void lm_launch(dim3 grid, hipStream_t stream, const bf16* x, int ld, int 
   constexpr int NP = 32 * NT, LDQ = NP + 8;
   const size_t lds = (size_t)(4 * LM_C * LDQ + 2 * NP * LM_LDT + LM_MTB * LM_LDT + 2 * LM_MTB * LDQ) * sizeof(uint16_t);
   // more than the default limit of dynamic LDS: asked for once per kernel
-  static const hipError_t asked = hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_attention_chunk_kernel<NT>),
+  static const hipError_t asked = hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_attention_chunk_kernel<NT, VEC>),
                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   (void)asked;
-  linear_attention_chunk_kernel<NT><<<grid, 256, lds, stream>>>(x, ld, oq, ok, ov, act, cos_t, sin_t, rd, key_scale,
+  linear_attention_chunk_kernel<NT, VEC><<<grid, 256, lds, stream>>>(x, ld, oq, ok, ov, act, cos_t, sin_t, rd, key_scale,
                                                                 decay, state, q_start, slots, positions, out, H, n, m,
                                                                 min_len);
 }
@@ -252,13 +351,20 @@ extern "C" int gs_linear_attention_chunks(const void* x, int ld, int oq, int ok,
   GS_REQUIRE(act == 0 || act == 1, "linear_attention_chunks: unknown activation %d", act);
   if (nseq == 0) return 0;
   dim3 grid(nseq, H, (m + LM_MTB - 1) / LM_MTB);
-#define LM_RUN(NT)                                                                                                   \
-  lm_launch<NT>(grid, stream, (const bf16*)x, ld, oq, ok, ov, act, cos_t, sin_t, rd, key_scale, decay, state, q_start, \
-                slots, positions, out, H, n, m, min_len)
-  if (n <= 32) LM_RUN(1);
-  else if (n <= 64) LM_RUN(2);
-  else if (n <= 96) LM_RUN(3);
-  else LM_RUN(4);
+  // rows as 16-byte pieces where every piece is whole and aligned, a turn's partner piece included
+  const bool vec = n % 8 == 0 && m % 8 == 0 && ld % 8 == 0 && oq % 8 == 0 && ok % 8 == 0 && ov % 8 == 0 && rd % 16 == 0 &&
+                   ((uintptr_t)x & 15) == 0 && ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0;
+#define LM_RUN(NT)                                                                                                        \
+  if (vec)                                                                                                                \
+    lm_launch<NT, true>(grid, stream, (const bf16*)x, ld, oq, ok, ov, act, cos_t, sin_t, rd, key_scale, decay, state,     \
+                        q_start, slots, positions, out, H, n, m, min_len);                                                \
+  else                                                                                                                    \
+    lm_launch<NT, false>(grid, stream, (const bf16*)x, ld, oq, ok, ov, act, cos_t, sin_t, rd, key_scale, decay, state,    \
+                         q_start, slots, positions, out, H, n, m, min_len)
+  if (n <= 32) { LM_RUN(1); }
+  else if (n <= 64) { LM_RUN(2); }
+  else if (n <= 96) { LM_RUN(3); }
+  else { LM_RUN(4); }
 #undef LM_RUN
   GS_LAUNCH_CHECK("linear_attention_chunks");
   return 0;

@@ -206,3 +206,44 @@ extern "C" int gs_qknorm_rope_kv(void* qkv, int dtype, const float* qw, const fl
   GS_LAUNCH_CHECK("qknorm_rope_kv");
   return 0;
 }
+
+// Rows of heads turned in place by their tokens' positions, backwards with sign < 0: x (T, nh, w), every head over its
+// whole width, pairs (i, i + w/2) or, with `interleaved`, (2i, 2i + 1); tables (max_position, w/2).  What attention
+// over values that were cached turned needs at its end: each head's sum turned back by the query's position.
+template <typename T>
+__global__ void turn_heads_kernel(T* __restrict__ x, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                  const int* __restrict__ positions, int interleaved, float sign, long units, int nh, int w) {
+  const int lane = threadIdx.x & 63;
+  const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (unit >= units) return;
+  const int t = (int)(unit / nh);
+  T* row = x + (size_t)unit * w;
+  const int half = w >> 1;
+  const float* cr = cos_t + (size_t)positions[t] * half;
+  const float* sr = sin_t + (size_t)positions[t] * half;
+  for (int i = lane; i < half; i += 64) {
+    const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+    const float a = to_f32(row[ia]), b = to_f32(row[ib]);
+    const float c = cr[i], s = sign * sr[i];
+    row[ia] = from_f32<T>(a * c - b * s);
+    row[ib] = from_f32<T>(a * s + b * c);
+  }
+}
+
+extern "C" int gs_turn_heads(void* x, int dtype, const float* cos_t, const float* sin_t, int max_position,
+                             const int* positions, int interleaved, float sign, int ntok, int nh, int w,
+                             hipStream_t stream) {
+  GS_REQUIRE(ntok >= 0 && nh > 0 && w > 0 && w % 2 == 0, "turn_heads: bad sizes T=%d nh=%d w=%d", ntok, nh, w);
+  GS_REQUIRE(cos_t && sin_t && max_position > 0, "turn_heads: no tables");
+  if (ntok == 0) return 0;
+  const long units = (long)ntok * nh;
+  const int blocks = gs_ceil_div(units, 4);
+  if (dtype == GS_F32)
+    turn_heads_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, cos_t, sin_t, positions, interleaved, sign, units, nh, w);
+  else if (dtype == GS_BF16)
+    turn_heads_kernel<bf16><<<blocks, 256, 0, stream>>>((bf16*)x, cos_t, sin_t, positions, interleaved, sign, units, nh, w);
+  else
+    GS_REQUIRE(false, "turn_heads: unknown dtype %d", dtype);
+  GS_LAUNCH_CHECK("turn_heads");
+  return 0;
+}

@@ -959,9 +959,26 @@ def attention_prefill_supports(nh: int, nkv: int, d: int) -> bool:
     return bool(lib().gs_attention_prefill_supports(c_int(nh), c_int(nkv), c_int(d)))
 
 
+def turn_heads(x, cos, sin, positions, nh: int, w: int, sign: float = 1.0, layout: str = "half") -> torch.Tensor:
+    """``x (T, nh w)`` in place: every head turned over its whole width by its token's position (``sign`` < 0:
+    backwards); tables ``(P, w/2)``."""
+    _dev(x, cos, sin, positions)
+    T = x.shape[0]
+    _need(x.dim() == 2 and x.shape[1] == nh * w, "turn_heads: rows (T, nh w)")
+    _value_tables(cos, sin, w)
+    _need(cos is not None, "turn_heads: no tables")
+    _need(layout in ROPE_LAYOUTS, f"turn_heads: pairs are laid out 'half' or 'interleaved', not {layout!r}")
+    _i32(positions, T, "positions")
+    _check(lib().gs_turn_heads(_p(x), c_int(_dt(x)), _p(cos), _p(sin), c_int(cos.shape[0]), _p(positions),
+                               c_int(1 if layout == "interleaved" else 0), c_float(sign), c_int(T), c_int(nh), c_int(w),
+                               _stream()))
+    return x
+
+
 def attention_prefill(q, q_stride, kcache, vcache, positions, tiles, block_table, page_size, window, scale, nh, nkv, d,
-                      ntok, out: torch.Tensor = None, tile_rows: int = 16) -> torch.Tensor:
-    """Causal GQA of many queries per sequence on the matrix cores (bfloat16).
+                      ntok, out: torch.Tensor = None, tile_rows: int = 16, chunk: int = None, sink: bool = False) -> torch.Tensor:
+    """Causal GQA of many queries per sequence on the matrix cores (bfloat16).  ``chunk``: a query sees only the keys
+    of its own run of ``chunk`` positions; ``sink``: one more term ``exp(0)`` in the softmax's denominator.
 
     ``tiles``: int32 ``(3, ntiles)``: sequence, first row and number of rows (at most ``tile_rows``, 16 or
     32) of each tile of consecutive queries of one sequence.
@@ -982,7 +999,8 @@ def attention_prefill(q, q_stride, kcache, vcache, positions, tiles, block_table
     _check(lib().gs_attention_prefill(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(tiles[0]),
                                       _p(tiles[1]), _p(tiles[2]), c_int(nt), _p(block_table),
                                       c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0), c_float(scale),
-                                      _p(out), c_int(nh), c_int(nkv), c_int(d), c_int(tile_rows), _stream()))
+                                      _p(out), c_int(nh), c_int(nkv), c_int(d), c_int(tile_rows), c_int(chunk or 0),
+                                      c_int(1 if sink else 0), _stream()))
     return out
 
 

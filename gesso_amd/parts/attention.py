@@ -210,8 +210,20 @@ class Attention(Part):
 
     def _attend_general(self, q, q_stride, ctx, cache) -> torch.Tensor:
         """Attention with values of their own width, runs of positions, a sink term or turned values: ``(T, nh * vd)``."""
-        s, ops, vp = self.spec, self.rt.ops, self.value_position
+        s, rt, ops, vp = self.spec, self.rt, self.rt.ops, self.value_position
         layout = getattr(vp, "layout", "half") if vp is not None else "half"
+        nh, nkv, d = s.n_heads, s.n_kv_heads, s.head_dim
+        if (q.dtype == torch.bfloat16 and not ctx.all_single and self.value_dim == d and cache.page_size >= 2
+                and q_stride % 8 == 0 and ops.attention_prefill_supports(nh, nkv, d) and ctx.recording is None):
+            # prompt portions whose values are as wide as their keys: the kernel on the matrix cores, which knows runs
+            # and the sink; the heads' sums are turned back afterwards
+            rows = 32 if ctx.max_q_len >= 64 and nh // nkv <= 4 else 16
+            out = ops.attention_prefill(q, q_stride, cache.k, cache.v, ctx.positions, ctx.query_tiles(rows, 0),
+                                        cache.block_table, cache.page_size, s.window, self.scale, nh, nkv, d, ctx.T,
+                                        tile_rows=rows, chunk=self.chunk, sink=self.sink)
+            if vp is not None:
+                ops.turn_heads(out, vp.cos, vp.sin, ctx.positions, nh, d, sign=-1.0, layout=layout)
+            return out
         return ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token, cache.block_table,
                                      cache.page_size, s.window, self.scale, s.n_heads, s.n_kv_heads, s.head_dim, ctx.T,
                                      vd=self.value_dim, chunk=self.chunk, sink=self.sink,

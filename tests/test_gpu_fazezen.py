@@ -244,7 +244,7 @@ def tables(dims, base, P_max, freqs=None):
 
 
 def attention_case(ops, dtype, nh, nkv, d, vd, rd, chunk, T, page_size, seed, sink=True, turned=True, boost=None,
-                   single_from=None, norm=True):
+                   single_from=None, norm=True, cores=False):
     """Random q | k | v rows of one sequence through the cache write (head norms, turns, turned values) and attention
     over shuffled pages; the plain implementation's result beside it.  ``boost = (query position, key position)``: that
     key is made to stand out for that query.  ``single_from``: the rows from there on go one token a launch."""
@@ -277,6 +277,14 @@ def attention_case(ops, dtype, nh, nkv, d, vd, rd, chunk, T, page_size, seed, si
         seq = torch.zeros(b - a, dtype=torch.int32, device=DEV)
         ops.qknorm_rope_kv(part, dev(qw), dev(kw), 1e-5, cos, sin, rd, i32(pos[a:b]), seq, bt, page_size, kc, vc, nh, nkv, d,
                            vd=vd, vcos=vcos, vsin=vsin)
+        if cores and b - a > 1:
+            # the kernel on the matrix cores, in tiles of 16 queries, and the heads' sums turned back afterwards
+            tiles = torch.tensor([[0] * len(range(0, b - a, 16)), list(range(0, b - a, 16)),
+                                  [min(16, b - a - r) for r in range(0, b - a, 16)]], dtype=torch.int32, device=DEV)
+            o = ops.attention_prefill(part, width, kc, vc, i32(pos[a:b]), tiles, bt, page_size, None, 0.3, nh, nkv, d, b - a,
+                                      chunk=chunk, sink=sink)
+            outs.append(ops.turn_heads(o, vcos, vsin, i32(pos[a:b]), nh, vd, sign=-1.0) if turned else o)
+            continue
         outs.append(ops.attention_generic(part, width, kc, vc, i32(pos[a:b]), seq, bt, page_size, None, 0.3, nh, nkv, d, b - a,
                                           vd=vd, chunk=chunk, sink=sink, vcos=vcos, vsin=vsin))
     got = torch.cat(outs).cpu().double()
@@ -314,6 +322,15 @@ def test_attention_within_runs_with_a_sink_and_turned_values(ops, dtype, nh, nkv
     assert float((got - want).abs().max()) <= tol(dtype, want, 2e-5, 2e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,rd,chunk,ps", [(4, 2, 64, 64, 64, 16), (2, 1, 128, 128, 128, 16), (8, 2, 32, 16, 24, 8),
+                                                  (3, 3, 64, 0, 7, 4), (2, 1, 64, 64, None, 16), (6, 1, 32, 32, 100, 16)])
+def test_attention_within_runs_on_the_matrix_cores(ops, nh, nkv, d, rd, chunk, ps):
+    got, want, _ = attention_case(ops, torch.bfloat16, nh, nkv, d, d, rd, chunk, 150, ps, seed=d + nh, cores=True)
+    assert float((got - want).abs().max()) <= tol(torch.bfloat16, want, 2e-5, 2e-2)
+    got, want, _ = attention_case(ops, torch.bfloat16, nh, nkv, d, d, rd, chunk, 70, ps, seed=d, sink=False, turned=False, cores=True)
+    assert float((got - want).abs().max()) <= tol(torch.bfloat16, want, 2e-5, 2e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("chunk,ps", [(24, 8), (21, 8), (32, 16), (None, 16)])
 def test_a_key_that_stands_out_is_found_at_the_edges_of_runs_and_pages_and_far_back(ops, dtype, chunk, ps):
@@ -343,6 +360,12 @@ def test_a_key_that_stands_out_is_found_at_the_edges_of_runs_and_pages_and_far_b
             alone = P.turn(v[kj:kj + 1, 0], [qi], P.frequencies(12, 1e4), sign=-1.0)[0]
             near = float((got[qi, :12] - alone).abs().max()) <= 0.05 * float(alone.abs().max())
             assert near == seen, (kj, single_from)
+        if dtype == torch.bfloat16:
+            # the same through the kernel on the matrix cores (keys and values 32 wide)
+            got, want, v = attention_case(ops, dtype, 2, 1, 32, 32, 16, chunk, T, ps, seed=kj, boost=(qi, kj), norm=False, cores=True)
+            assert float((got - want).abs().max()) <= tol(dtype, want, 3e-5, 3e-2), kj
+            alone = P.turn(v[kj:kj + 1, 0], [qi], P.frequencies(32, 1e4), sign=-1.0)[0]
+            assert (float((got[qi, :32] - alone).abs().max()) <= 0.05 * float(alone.abs().max())) == seen, kj
 
 
 # ------------------------------------------------------------------ the mixers alone, with their own caches
