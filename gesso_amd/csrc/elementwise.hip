@@ -611,14 +611,15 @@ extern "C" int gs_fill_rows(void* pool, int dtype, const int* ids, int n, long r
 
 // ------------------------------------------------------------------ two adds + two RMSNorms of one row
 
-// One block per row: x = res (+ d1) (+ d2), written back; out1 = x * inv_rms(x) * w1, out2 = x * inv_rms(x) * w2
-// (out2 and w2 may be absent).  The block of a layer whose mixer and feed-forward both read the same stream, each
+// One block per row: x = res (+ d1) (+ d2) (+ bias, one vector for all rows), written back; out1 = x * inv_rms(x) * w1,
+// out2 = x * inv_rms(x) * w2 (out2 and w2 may be absent).  The block of a layer whose mixer and feed-forward both read the same stream, each
 // through a norm of its own, needs the stream's row once for both; the two results of the layer before are added on
 // the way.  The row stays in registers or LDS between the passes: rows up to 8192 values, else it is read again.
 template <typename TD, typename TO>
 __global__ void add_rmsnorm_pair_kernel(float* __restrict__ res, const TD* __restrict__ d1, const TD* __restrict__ d2,
                                         const float* __restrict__ w1, const float* __restrict__ w2, float eps,
-                                        TO* __restrict__ out1, TO* __restrict__ out2, int H) {
+                                        TO* __restrict__ out1, TO* __restrict__ out2, int H,
+                                        const float* __restrict__ bias) {
   __shared__ float red[17];
   const int r = blockIdx.x;
   float* x = res + (size_t)r * H;
@@ -629,7 +630,8 @@ __global__ void add_rmsnorm_pair_kernel(float* __restrict__ res, const TD* __res
     float v = x[j];
     if (a) v += to_f32(a[j]);
     if (b) v += to_f32(b[j]);
-    if (a || b) x[j] = v;
+    if (bias) v += bias[j];
+    if (a || b || bias) x[j] = v;
     ss += v * v;
   }
   ss = block_sum(ss, red);
@@ -645,7 +647,7 @@ __global__ void add_rmsnorm_pair_kernel(float* __restrict__ res, const TD* __res
 
 extern "C" int gs_add_rmsnorm_pair(float* res, const void* d1, const void* d2, int delta_dtype, const float* w1,
                                    const float* w2, float eps, void* out1, void* out2, int out_dtype, int T, int H,
-                                   hipStream_t stream) {
+                                   const float* bias, hipStream_t stream) {
   GS_REQUIRE(T >= 0 && H > 0, "add_rmsnorm_pair: bad sizes rows=%d H=%d", T, H);
   GS_REQUIRE(eps > 0.f, "add_rmsnorm_pair: eps must be positive");
   GS_REQUIRE(w1 && out1 && ((w2 == nullptr) == (out2 == nullptr)), "add_rmsnorm_pair: a weight for every output");
@@ -653,7 +655,7 @@ extern "C" int gs_add_rmsnorm_pair(float* res, const void* d1, const void* d2, i
   const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
 #define GS_RUN(TD, TO)                                                                                             \
   add_rmsnorm_pair_kernel<TD, TO><<<T, threads, 0, stream>>>(res, (const TD*)d1, (const TD*)d2, w1, w2, eps,       \
-                                                              (TO*)out1, (TO*)out2, H)
+                                                              (TO*)out1, (TO*)out2, H, bias)
   if (delta_dtype == GS_F32 && out_dtype == GS_F32)
     GS_RUN(float, float);
   else if (delta_dtype == GS_BF16 && out_dtype == GS_BF16)

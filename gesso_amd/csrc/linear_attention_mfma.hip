@@ -10,8 +10,9 @@
 // state (transposed, 32 x n) stays in its accumulators from run to run.  Products are v_mfma_f32_32x32x16_bf16 with
 // float32 sums.  What the design holds in 32 bits (activated and turned q and k, the decayed scores, the state, the
 // decayed keys) enters the products as two bfloat16 terms, the value's rounding and the rounding of what is left, and
-// each product is three (hi hi + hi lo + lo hi): sixteen bits of every operand, the sums in float32.  Values enter as
-// one term (a projection with its activation).  Powers of the decay come from a table made by repeated multiplication.
+// each product is three (hi hi + hi lo + lo hi): sixteen bits of every operand, the sums in float32.  Values as they
+// come from their product are bfloat16 already and enter as one term; activated values as two, like the rest.  Powers
+// of the decay come from a table made by repeated multiplication.
 //
 // The scores are computed transposed (rows s, columns t), which leaves them, in a lane's registers, in the order in
 // which the next product takes its first operand, but for a permutation of the 16 inner indices of a step: slot q of
@@ -19,6 +20,15 @@
 // 8-byte reads).  No trip of the scores through LDS, no wait between the two products.
 //
 // Sequences shorter than `min_len` tokens are left alone (the token-by-token kernel takes them).
+//
+// One block a (sequence, head) walks the runs one after the other, which leaves most of the chip idle when a step
+// brings few long portions.  Then the portions are cut into segments of `seg_len` tokens and three launches do the
+// work (MODE): (1) every segment by a block of its own, from the request's state (the first segment) or from an empty
+// one, its outputs stored and its last state left in a workspace; (2) a light kernel goes through a sequence's
+// segments in order, S_start[p + 1] = d^len(p) S_start[p] + G[p], leaves every segment's first state in the workspace
+// and the last state in the request's slot; (3) every segment but the first adds what its first state gives its
+// tokens, d^(t + 1) q_t S_start, the first of the two terms of O above, with the state's decay from run to run kept
+// as one factor.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 lm_bf16x8_t;
@@ -40,12 +50,13 @@ __device__ __forceinline__ void lm_split(float v, uint16_t& hi, uint16_t& lo) {
   lo = f32_to_bf16(v - to_f32(h)).x;
 }
 
-template <int NT, bool VEC>
+template <int NT, bool VEC, int MODE>
 __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
     const bf16* __restrict__ x, int ld, int oq, int ok, int ov, int act, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int rd, float key_scale, const float* __restrict__ decay,
     float* __restrict__ state, const int* __restrict__ q_start, const int* __restrict__ slots,
-    const int* __restrict__ positions, float* __restrict__ out, int H, int n, int m, int min_len) {
+    const int* __restrict__ positions, float* __restrict__ out, int H, int n, int m, int min_len,
+    float* __restrict__ ws, int maxseg, int seg_len) {
   constexpr int NP = 32 * NT, LDQ = NP + 8;
   extern __shared__ __align__(16) uint16_t lm_lds[];
   uint16_t* Qh = lm_lds;  // [32][LDQ] each
@@ -55,18 +66,30 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
   uint16_t* KTh = Kl + LM_C * LDQ;  // [NP][LDT] each: decayed keys, transposed
   uint16_t* KTl = KTh + NP * LM_LDT;
   uint16_t* VT = KTl + NP * LM_LDT;      // [MTB][LDT]: values, transposed
-  uint16_t* STh = VT + LM_MTB * LM_LDT;  // [MTB][LDQ] each: the state, transposed
+  uint16_t* VTl = VT + LM_MTB * LM_LDT;  // the same: what the rounding of activated values left
+  uint16_t* STh = VTl + LM_MTB * LM_LDT;  // [MTB][LDQ] each: the state, transposed
   uint16_t* STl = STh + LM_MTB * LDQ;
   __shared__ float pw[LM_C + 1];
 
-  const int seq = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * LM_MTB;
-  const int t0 = q_start[seq], t1 = q_start[seq + 1];
+  const int seq = MODE == 0 ? blockIdx.x : blockIdx.x / maxseg, seg = MODE == 0 ? 0 : blockIdx.x % maxseg;
+  const int h = blockIdx.y, j0 = blockIdx.z * LM_MTB;
+  const int ts = q_start[seq];            // the sequence's first row of this step
+  int t0 = ts, t1 = q_start[seq + 1];
   if (t1 - t0 < min_len || t1 <= t0) return;
+  if (MODE != 0) {
+    if (MODE == 2 && seg == 0) return;    // the first segment started from the true state
+    t0 = ts + seg * seg_len;
+    if (t0 >= t1) return;
+    t1 = t1 < t0 + seg_len ? t1 : t0 + seg_len;
+  }
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
   const int jw = wave * 32;
   const bool live = j0 + jw < m;      // a wavefront whose columns all lie beyond m only helps staging
   const float d = decay[h];
-  float* S = state + (((size_t)slots[seq] * H + h) * n) * m;
+  // where the state comes from and goes to: the request's slot, or the segment's place in the workspace
+  float* W = MODE == 0 ? nullptr : ws + ((((size_t)seq * maxseg + seg) * H + h) * n) * m;
+  float* S = (MODE == 0 || (MODE == 1 && seg == 0)) ? state + (((size_t)slots[seq] * H + h) * n) * m : W;
+  const bool empty = MODE == 1 && seg > 0;
   if (tid == 0) {
     float p = 1.f;
     for (int e = 0; e <= LM_C; ++e) {
@@ -80,9 +103,10 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int i = it * 32 + l32, j = j0 + jw + 8 * (e / 4) + 4 * half + e % 4;
-      acc_s[it][e] = (i < n && j < m) ? S[(size_t)i * m + j] : 0.f;
+      acc_s[it][e] = (!empty && i < n && j < m) ? S[(size_t)i * m + j] : 0.f;
     }
   const int hr = rd >> 1;
+  float cum = 1.f;        // MODE 2: the state's decay over the runs gone by
 
   // VEC: a run's rows come as 16-byte pieces (eight features of one token), all of a thread's pieces asked for at once
   // and, from the second run on, while the run before is still being computed.  Piece u of a thread: token
@@ -91,7 +115,7 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
   // multiple of eight).  Values: piece (tid + 256 u) % 32 -> token, / 32 -> eight columns.
   constexpr int UQ = (LM_C * NP / 8 + 255) / 256, UV = LM_C * LM_MTB / 8 / 256;
   uint4 rq[UQ], rk[UQ], rqo[UQ], rko[UQ], rv[UV];
-  const int pos0 = positions[t0];
+  const int pos0 = positions[ts];
   auto fetch = [&](int tb, int nb) {
     if constexpr (VEC) {
 #pragma unroll
@@ -101,11 +125,11 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
         if (t < nb && i < n) {
           const bf16* row = x + (size_t)(tb + t) * ld;
           rq[u] = *reinterpret_cast<const uint4*>(row + oq + h * n + i);
-          rk[u] = *reinterpret_cast<const uint4*>(row + ok + h * n + i);
+          if (MODE != 2) rk[u] = *reinterpret_cast<const uint4*>(row + ok + h * n + i);
           if (i < rd) {
             const int other = i < hr ? i + hr : i - hr;
             rqo[u] = *reinterpret_cast<const uint4*>(row + oq + h * n + other);
-            rko[u] = *reinterpret_cast<const uint4*>(row + ok + h * n + other);
+            if (MODE != 2) rko[u] = *reinterpret_cast<const uint4*>(row + ok + h * n + other);
           }
         }
       }
@@ -113,7 +137,8 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
       for (int u = 0; u < UV; ++u) {
         const int piece = tid + 256 * u, t = piece % LM_C, c = (piece / LM_C) * 8;
         rv[u] = make_uint4(0, 0, 0, 0);
-        if (t < nb && j0 + c < m) rv[u] = *reinterpret_cast<const uint4*>(x + (size_t)(tb + t) * ld + ov + h * m + j0 + c);
+        if (MODE != 2 && t < nb && j0 + c < m)
+          rv[u] = *reinterpret_cast<const uint4*>(x + (size_t)(tb + t) * ld + ov + h * m + j0 + c);
       }
     }
   };
@@ -143,8 +168,8 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
         const bool turned = t < nb && i < rd, low = i < hr;
         float c8[8], s8[8];
         if (turned) {
-          const float* cr = cos_t + (size_t)(pos0 + tb - t0 + t) * hr + (low ? i : i - hr);
-          const float* sr = sin_t + (size_t)(pos0 + tb - t0 + t) * hr + (low ? i : i - hr);
+          const float* cr = cos_t + (size_t)(pos0 + tb - ts + t) * hr + (low ? i : i - hr);
+          const float* sr = sin_t + (size_t)(pos0 + tb - ts + t) * hr + (low ? i : i - hr);
           load8f(cr, c8);
           load8f(sr, s8);
         }
@@ -178,7 +203,7 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
         float v8[8];
         eight(rv[u], v8);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) VT[(c + e) * LM_LDT + t] = f32_to_bf16(lm_act(v8[e], act)).x;
+        for (int e = 0; e < 8; ++e) lm_split(lm_act(v8[e], act), VT[(c + e) * LM_LDT + t], VTl[(c + e) * LM_LDT + t]);
       }
     } else {
       for (int idx = tid; idx < LM_C * NP; idx += 256) {
@@ -209,10 +234,10 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
         const int t = idx / LM_MTB, c = idx - t * LM_MTB;
         const int j = j0 + c;
         const float v = (t < nb && j < m) ? lm_act(to_f32(x[(size_t)(tb + t) * ld + ov + h * m + j]), act) : 0.f;
-        VT[c * LM_LDT + t] = f32_to_bf16(v).x;
+        lm_split(v, VT[c * LM_LDT + t], VTl[c * LM_LDT + t]);
       }
     }
-    if (live) {
+    if (live && (MODE != 2 || tb == t0)) {
 #pragma unroll
       for (int it = 0; it < NT; ++it)
 #pragma unroll
@@ -225,6 +250,32 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
     if (tb + LM_C < t1) fetch(tb + LM_C, t1 - tb - LM_C < LM_C ? t1 - tb - LM_C : LM_C);   // the next run's rows, meanwhile
     if (!live) continue;
 
+    if constexpr (MODE == 2) {
+      lm_f32x16_t o2;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o2[e] = 0.f;
+      const int ro2 = l32 * LDQ + half * 8, so2 = (jw + l32) * LDQ + half * 8;
+#pragma unroll
+      for (int ks = 0; ks < NP / 16; ++ks) {
+        const lm_bf16x8_t qh8 = *reinterpret_cast<const lm_bf16x8_t*>(Qh + ro2 + ks * 16);
+        const lm_bf16x8_t ql8 = *reinterpret_cast<const lm_bf16x8_t*>(Ql + ro2 + ks * 16);
+        const lm_bf16x8_t sh8 = *reinterpret_cast<const lm_bf16x8_t*>(STh + so2 + ks * 16);
+        const lm_bf16x8_t sl8 = *reinterpret_cast<const lm_bf16x8_t*>(STl + so2 + ks * 16);
+        o2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qh8, sh8, o2, 0, 0, 0);
+        o2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qh8, sl8, o2, 0, 0, 0);
+        o2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ql8, sh8, o2, 0, 0, 0);
+      }
+      const int j2 = j0 + jw + l32;
+      if (j2 < m) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int t = 8 * (e / 4) + 4 * half + e % 4;
+          if (t < nb) out[((size_t)(tb + t) * H + h) * m + j2] += o2[e] * (pw[t + 1] * cum);
+        }
+      }
+      cum *= pw[nb];
+      continue;
+    }
     // scores, transposed: rows s, columns t
     lm_f32x16_t at;
 #pragma unroll
@@ -281,6 +332,17 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
       }
       o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[k2], v8, o, 0, 0, 0);
       o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[k2], v8, o, 0, 0, 0);
+      if (act) {      // activated values have a second term
+        const lm_bf16x4_t w0 = *reinterpret_cast<const lm_bf16x4_t*>(VTl + vo + 16 * k2 + 4 * half);
+        const lm_bf16x4_t w1 = *reinterpret_cast<const lm_bf16x4_t*>(VTl + vo + 16 * k2 + 8 + 4 * half);
+        lm_bf16x8_t w8;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          w8[q] = w0[q];
+          w8[4 + q] = w1[q];
+        }
+        o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[k2], w8, o, 0, 0, 0);
+      }
     }
     {
       const int j = j0 + jw + l32;
@@ -306,6 +368,10 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
         const lm_bf16x8_t kl8 = *reinterpret_cast<const lm_bf16x8_t*>(KTl + ko);
         acc_s[it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v8, kh8, acc_s[it], 0, 0, 0);
         acc_s[it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v8, kl8, acc_s[it], 0, 0, 0);
+        if (act) {
+          const lm_bf16x8_t w8 = *reinterpret_cast<const lm_bf16x8_t*>(VTl + vo + 16 * k2 + 8 * half);
+          acc_s[it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w8, kh8, acc_s[it], 0, 0, 0);
+        }
       }
     }
   }
@@ -314,24 +380,56 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int i = it * 32 + l32, j = j0 + jw + 8 * (e / 4) + 4 * half + e % 4;
-      if (i < n && j < m) S[(size_t)i * m + j] = acc_s[it][e];
+      if (MODE != 2 && i < n && j < m) (MODE == 0 ? S : W)[(size_t)i * m + j] = acc_s[it][e];
     }
 }
 
-template <int NT, bool VEC>
+// Pass (2) of the three: one thread per (sequence, head, element of the state), on its own through the segments.
+__global__ void linear_attention_combine_kernel(const float* __restrict__ decay, float* __restrict__ state,
+                                                const int* __restrict__ q_start, const int* __restrict__ slots,
+                                                float* __restrict__ ws, int H, int n, int m, int min_len, int maxseg,
+                                                int seg_len) {
+  const int seq = blockIdx.x, h = blockIdx.y;
+  const int len = q_start[seq + 1] - q_start[seq];
+  if (len < min_len || len <= 0) return;
+  const int nseg = (len + seg_len - 1) / seg_len;
+  const float d = decay[h];
+  float dfull = 1.f, dlast = 1.f;                     // d^seg_len and d^(the last segment's length), as the table's powers
+  const int last = len - (nseg - 1) * seg_len;
+  for (int e = 0; e < seg_len; ++e) {
+    dfull *= d;
+    if (e < last) dlast *= d;
+  }
+  const size_t per = (size_t)n * m;
+  float* S = state + ((size_t)slots[seq] * H + h) * per;
+  const size_t idx = (size_t)blockIdx.z * blockDim.x + threadIdx.x;
+  if (idx < per) {
+    float cur = ws[(((size_t)seq * maxseg) * H + h) * per + idx];
+    for (int p = 1; p < nseg; ++p) {
+      float* g = ws + (((size_t)seq * maxseg + p) * H + h) * per + idx;
+      const float own = *g;
+      *g = cur;                                       // the state the segment starts from
+      cur = (p == nseg - 1 ? dlast : dfull) * cur + own;
+    }
+    S[idx] = cur;
+  }
+}
+
+template <int NT, bool VEC, int MODE>
 static void lm_launch(dim3 grid, hipStream_t stream, const bf16* x, int ld, int oq, int ok, int ov, int act,
                       const float* cos_t, const float* sin_t, int rd, float key_scale, const float* decay, float* state,
                       const int* q_start, const int* slots, const int* positions, float* out, int H, int n, int m,
-                      int min_len) {
+                      int min_len, float* ws, int maxseg, int seg_len) {
   constexpr int NP = 32 * NT, LDQ = NP + 8;
-  const size_t lds = (size_t)(4 * LM_C * LDQ + 2 * NP * LM_LDT + LM_MTB * LM_LDT + 2 * LM_MTB * LDQ) * sizeof(uint16_t);
+  const size_t lds = (size_t)(4 * LM_C * LDQ + 2 * NP * LM_LDT + 2 * LM_MTB * LM_LDT + 2 * LM_MTB * LDQ) * sizeof(uint16_t);
   // more than the default limit of dynamic LDS: asked for once per kernel
-  static const hipError_t asked = hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_attention_chunk_kernel<NT, VEC>),
+  static const hipError_t asked = hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_attention_chunk_kernel<NT, VEC, MODE>),
                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   (void)asked;
-  linear_attention_chunk_kernel<NT, VEC><<<grid, 256, lds, stream>>>(x, ld, oq, ok, ov, act, cos_t, sin_t, rd, key_scale,
-                                                                decay, state, q_start, slots, positions, out, H, n, m,
-                                                                min_len);
+  linear_attention_chunk_kernel<NT, VEC, MODE><<<grid, 256, lds, stream>>>(x, ld, oq, ok, ov, act, cos_t, sin_t, rd,
+                                                                           key_scale, decay, state, q_start, slots,
+                                                                           positions, out, H, n, m, min_len, ws, maxseg,
+                                                                           seg_len);
 }
 
 extern "C" int gs_linear_attention_chunks_max_key() { return 128; }
@@ -340,7 +438,10 @@ extern "C" int gs_linear_attention_chunks(const void* x, int ld, int oq, int ok,
                                           const float* sin_t, int rd, int max_position, float key_scale,
                                           const float* decay, float* state, const int* q_start, const int* slots,
                                           const int* positions, float* out, int nseq, int H, int n, int m, int min_len,
-                                          hipStream_t stream) {
+                                          float* ws, int maxseg, int seg_len, hipStream_t stream) {
+  GS_REQUIRE(maxseg >= 0 && (maxseg == 0 || (ws && seg_len > 0 && seg_len % LM_C == 0)),
+             "linear_attention_chunks: segments of %d tokens (whole runs of %d) with a workspace", seg_len, LM_C);
+  GS_REQUIRE(maxseg == 0 || (long)nseq * maxseg <= 0x7fffffffL, "linear_attention_chunks: too many segments");
   GS_REQUIRE(nseq >= 0 && H > 0 && n > 0 && m > 0, "linear_attention_chunks: bad sizes nseq=%d H=%d n=%d m=%d", nseq, H, n, m);
   GS_REQUIRE(n <= 128, "linear_attention_chunks: keys of %d features, the kernel holds up to 128", n);
   GS_REQUIRE(H <= 65535 && (m + LM_MTB - 1) / LM_MTB <= 65535, "linear_attention_chunks: too many heads or value columns");
@@ -350,22 +451,32 @@ extern "C" int gs_linear_attention_chunks(const void* x, int ld, int oq, int ok,
              "linear_attention_chunks: q, k or v lie outside the rows of %d", ld);
   GS_REQUIRE(act == 0 || act == 1, "linear_attention_chunks: unknown activation %d", act);
   if (nseq == 0) return 0;
-  dim3 grid(nseq, H, (m + LM_MTB - 1) / LM_MTB);
+  dim3 grid(maxseg > 0 ? nseq * maxseg : nseq, H, (m + LM_MTB - 1) / LM_MTB);
   // rows as 16-byte pieces where every piece is whole and aligned, a turn's partner piece included
   const bool vec = n % 8 == 0 && m % 8 == 0 && ld % 8 == 0 && oq % 8 == 0 && ok % 8 == 0 && ov % 8 == 0 && rd % 16 == 0 &&
                    ((uintptr_t)x & 15) == 0 && ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0;
-#define LM_RUN(NT)                                                                                                        \
-  if (vec)                                                                                                                \
-    lm_launch<NT, true>(grid, stream, (const bf16*)x, ld, oq, ok, ov, act, cos_t, sin_t, rd, key_scale, decay, state,     \
-                        q_start, slots, positions, out, H, n, m, min_len);                                                \
-  else                                                                                                                    \
-    lm_launch<NT, false>(grid, stream, (const bf16*)x, ld, oq, ok, ov, act, cos_t, sin_t, rd, key_scale, decay, state,    \
-                         q_start, slots, positions, out, H, n, m, min_len)
+#define LM_ARGS                                                                                                      \
+  grid, stream, (const bf16*)x, ld, oq, ok, ov, act, cos_t, sin_t, rd, key_scale, decay, state, q_start, slots, positions, \
+      out, H, n, m, min_len, ws, maxseg, seg_len
+#define LM_MODES(NT, V)                                                                                              \
+  if (maxseg == 0) {                                                                                                 \
+    lm_launch<NT, V, 0>(LM_ARGS);                                                                                    \
+  } else {                                                                                                           \
+    lm_launch<NT, V, 1>(LM_ARGS);                                                                                    \
+    linear_attention_combine_kernel<<<dim3(nseq, H, (n * m + 255) / 256), 256, 0, stream>>>(                          \
+        decay, state, q_start, slots, ws, H, n, m, min_len, maxseg, seg_len);                                        \
+    if (maxseg > 1) lm_launch<NT, V, 2>(LM_ARGS);                                                                    \
+  }
+#define LM_RUN(NT)                 \
+  if (vec) { LM_MODES(NT, true) }  \
+  else { LM_MODES(NT, false) }
   if (n <= 32) { LM_RUN(1); }
   else if (n <= 64) { LM_RUN(2); }
   else if (n <= 96) { LM_RUN(3); }
   else { LM_RUN(4); }
 #undef LM_RUN
+#undef LM_MODES
+#undef LM_ARGS
   GS_LAUNCH_CHECK("linear_attention_chunks");
   return 0;
 }

@@ -390,7 +390,8 @@ LINEAR_ATTENTION_CHUNKS_MAX_KEY = 128
 
 def linear_attention_scan(x, oq: int, ok: int, ov: int, H: int, n: int, m: int, decay, state, q_start, slots, positions,
                           nseq: int, activation=None, cos=None, sin=None, rotary_dim: int = 0, key_scale: float = 1.0,
-                          out: torch.Tensor = None, below: int = 0, chunks_from: int = 0) -> torch.Tensor:
+                          out: torch.Tensor = None, below: int = 0, chunks_from: int = 0, segment: int = 0,
+                          longest: int = 0) -> torch.Tensor:
     """Linear attention through a fading state: per sequence and head ``S <- decay_h S + k_t v_t^T``, ``o_t = S^T q_t``.
 
     ``x (T, ld)`` holds q of head h at columns ``[oq + h n, ...)``, k at ``[ok + h n, ...)``, v at ``[ov + h m, ...)``;
@@ -400,7 +401,9 @@ def linear_attention_scan(x, oq: int, ok: int, ov: int, H: int, n: int, m: int, 
 
     ``below`` > 0: only the sequences that bring fewer tokens than that (the rows of the others are left as they are).
     ``chunks_from`` > 0: the kernel on the matrix cores instead (bfloat16 rows, keys up to
-    ``LINEAR_ATTENTION_CHUNKS_MAX_KEY`` wide), for the sequences that bring at least that many tokens."""
+    ``LINEAR_ATTENTION_CHUNKS_MAX_KEY`` wide), for the sequences that bring at least that many tokens; with
+    ``segment`` > 0 (a multiple of 32) those sequences are cut into segments of that many tokens, each a block of its
+    own, in three launches (``longest``: the most tokens a sequence brings)."""
     _dev(x, decay, state, q_start, slots, positions, cos, sin, out)
     _need(x.dim() == 2, "linear_attention: rows (T, ld)")
     T, ld = x.shape
@@ -423,11 +426,17 @@ def linear_attention_scan(x, oq: int, ok: int, ov: int, H: int, n: int, m: int, 
     if chunks_from > 0:
         _need(x.dtype == torch.bfloat16 and n <= LINEAR_ATTENTION_CHUNKS_MAX_KEY,
               "linear_attention: the kernel on the matrix cores takes bfloat16 rows and keys up to 128 wide")
+        ws, maxseg = None, 0
+        if segment > 0:
+            _need(segment % 32 == 0 and longest > 0, "linear_attention: segments are whole runs of 32 tokens")
+            maxseg = -(-longest // segment)
+            ws = torch.empty(nseq * maxseg * H * n * m, dtype=torch.float32, device=x.device)
         _check(lib().gs_linear_attention_chunks(_p(x), c_int(ld), c_int(oq), c_int(ok), c_int(ov), c_int(_ACTS[activation]),
                                                 _p(cos) if rotary_dim else None, _p(sin) if rotary_dim else None,
                                                 c_int(rotary_dim), c_int(max_pos), c_float(key_scale), _p(decay), _p(state),
                                                 _p(q_start), _p(slots), _p(positions), _p(out), c_int(nseq), c_int(H),
-                                                c_int(n), c_int(m), c_int(chunks_from), _stream()))
+                                                c_int(n), c_int(m), c_int(chunks_from), _p(ws), c_int(maxseg),
+                                                c_int(segment), _stream()))
         return out
     _check(lib().gs_linear_attention_scan(_p(x), c_int(_dt(x)), c_int(ld), c_int(oq), c_int(ok), c_int(ov),
                                           c_int(_ACTS[activation]), _p(cos) if rotary_dim else None,
@@ -455,13 +464,14 @@ def gated_outnorm(o, gate_rows, og: int, weight, eps: float, H: int, m: int, joi
     return out
 
 
-def add_rmsnorm_pair(res, d1, d2, w1, w2, eps: float, out_dtype):
-    """``res += d1 + d2`` (each where given), then ``(rmsnorm(res) * w1, rmsnorm(res) * w2)``; ``w2`` None: one result."""
-    _dev(res, d1, d2, w1, w2)
+def add_rmsnorm_pair(res, d1, d2, w1, w2, eps: float, out_dtype, bias=None):
+    """``res += d1 + d2 + bias`` (each where given; ``bias (H,)`` float32 is added to every row), then
+    ``(rmsnorm(res) * w1, rmsnorm(res) * w2)``; ``w2`` None: one result."""
+    _dev(res, d1, d2, w1, w2, bias)
     _need(res.dtype == torch.float32 and res.dim() == 2, "add_rmsnorm_pair: the residual stream is float32 (T, H)")
     T, H = res.shape
-    for w in (w1, w2):
-        _need(w is None or (w.dtype == torch.float32 and w.shape == (H,)), "add_rmsnorm_pair: weights must be float32 (H,)")
+    for w in (w1, w2, bias):
+        _need(w is None or (w.dtype == torch.float32 and w.shape == (H,)), "add_rmsnorm_pair: weights and bias must be float32 (H,)")
     _need(w1 is not None, "add_rmsnorm_pair: a first weight")
     ds = [d for d in (d1, d2) if d is not None]
     for d in ds:
@@ -470,7 +480,7 @@ def add_rmsnorm_pair(res, d1, d2, w1, w2, eps: float, out_dtype):
     out2 = torch.empty((T, H), dtype=out_dtype, device=res.device) if w2 is not None else None
     _check(lib().gs_add_rmsnorm_pair(_p(res), _p(ds[0]) if ds else None, _p(ds[1]) if len(ds) > 1 else None,
                                      c_int(_dt(ds[0]) if ds else _dt(out1)), _p(w1), _p(w2), c_float(eps), _p(out1),
-                                     _p(out2), c_int(_dt(out1)), c_int(T), c_int(H), _stream()))
+                                     _p(out2), c_int(_dt(out1)), c_int(T), c_int(H), _p(bias), _stream()))
     return out1, out2
 
 

@@ -128,14 +128,20 @@ class ParallelBlock(PreNormBlock):
         with rt.stage("norm"):
             second = self.ffn_norm if self.ffn is not None else None
             x1, x2 = ops.add_rmsnorm_pair(stream.res, held[0], held[1], self.mixer_norm.weight,
-                                          None if second is None else second.weight, self.mixer_norm.spec.eps, rt.dtype)
-        stream.pending = stream.ssq = stream.xs = stream.xs_for = stream.normed = stream.rows = None
+                                          None if second is None else second.weight, self.mixer_norm.spec.eps, rt.dtype,
+                                          bias=stream.bias)
+        stream.pending = stream.ssq = stream.xs = stream.xs_for = stream.normed = stream.rows = stream.bias = None
         with rt.stage(getattr(self.mixer, "stage", "mixer")):
             a = rt.dense(self.mixer.forward(x1, ctx, cache))
         b = None
         if self.ffn is not None:
             with rt.stage(getattr(self.ffn, "stage", "ffn")):
-                b = rt.dense(self.ffn.forward(x2, ctx))
+                if getattr(self.ffn, "defers_bias", False):
+                    # the last product's bias waits for the pass that adds the product to the stream
+                    b, stream.bias = self.ffn.forward(x2, ctx, defer_bias=True)
+                    b = rt.dense(b)
+                else:
+                    b = rt.dense(self.ffn.forward(x2, ctx))
         stream.pending = (a, b)
 
     @property

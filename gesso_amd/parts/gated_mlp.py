@@ -42,11 +42,17 @@ class GatedMLP(Part):
             self.b_gu = torch.cat([tensors["gate.bias"], tensors["up.bias"]], 0).contiguous()
             self.b_down = tensors["down.bias"]
 
-    def forward(self, x, ctx):
+    defers_bias = True
+
+    def forward(self, x, ctx, defer_bias: bool = False):
+        """``defer_bias``: returns ``(product without the last bias, that bias or None)``, for a block that adds the
+        bias where it adds the product."""
         rt = self.rt
         with rt.stage("ffn_gateup"):
             gu = rt.linear(rt.dense(x), self.w_gu)
             a = rt.ops.gated_act(gu, self.b_gu, self.spec.activation, rt.dtype)
+        if defer_bias:
+            return rt.linear(a, self.w_down), self.b_down
         return rt.linear(a, self.w_down, self.b_down)
 
 

@@ -24,6 +24,7 @@ class LinearAttention(Part):
     graph_safe = True
     stage, out_stage = "linear_mixer", "linear_out"
     RUNS_FROM = 8       # sequences that bring at least this many tokens to a step go to the kernel on the matrix cores
+    SEGMENT = 128       # tokens of a segment where long portions are cut to fill the chip
 
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
@@ -76,7 +77,11 @@ class LinearAttention(Part):
                     and n <= ops.LINEAR_ATTENTION_CHUNKS_MAX_KEY and ctx.max_q_len >= self.RUNS_FROM)
             if runs:
                 # prompt portions 32 tokens at a time on the matrix cores; what brings fewer tokens, token by token
-                o = ops.linear_attention_scan(*args, chunks_from=self.RUNS_FROM, **kw)
+                # few long portions: cut into segments that run side by side (a block a sequence and head would leave
+                # most of the chip idle)
+                blocks = sum(1 for L in ctx.q_lens if L >= self.RUNS_FROM) * H * -(-m // 128)
+                cut = self.SEGMENT if ctx.max_q_len >= 2 * self.SEGMENT and blocks < rt.compute_units else 0
+                o = ops.linear_attention_scan(*args, chunks_from=self.RUNS_FROM, segment=cut, longest=ctx.max_q_len, **kw)
                 if min(ctx.q_lens) < self.RUNS_FROM:
                     ops.linear_attention_scan(*args, below=self.RUNS_FROM, out=o, **kw)
             else:

@@ -25,7 +25,7 @@ class ResidualStream:
     in bfloat16, and the norm's consumer needs no norm pass at all.  ``xs_for`` is the norm ``xs`` was made for.
     """
 
-    __slots__ = ("res", "pending", "ssq", "xs", "xs_for", "following", "normed", "rows")
+    __slots__ = ("res", "pending", "ssq", "xs", "xs_for", "following", "normed", "rows", "bias")
 
     def __init__(self, res, pending=None, ssq=None, xs=None, xs_for=None):
         self.res = res
@@ -35,6 +35,8 @@ class ResidualStream:
         self.following = None
         self.normed = None            # the rows normed for ``xs_for``, where the last push made them
         self.rows = None              # the stream itself in the activation type, where the last writer left it
+        self.bias = None              # a float32 vector still to be added to every row (a last product's bias, left
+                                      # for the pass that adds the product itself)
 
     def push(self, out, rt, next_norm=None) -> None:
         from .runtime import DeferredLinear
@@ -68,6 +70,10 @@ class ResidualStream:
                 if delta is not None:
                     rt.ops.residual_add(self.res, delta)      # (a parallel block leaves two results)
             self.pending, self.ssq = None, None
+            self.xs = self.xs_for = self.normed = self.rows = None
+        if self.bias is not None:
+            rt.ops.add_bias(self.res, self.bias, torch.float32, out=self.res)
+            self.bias, self.ssq = None, None
             self.xs = self.xs_for = self.normed = self.rows = None
 
 
@@ -104,7 +110,7 @@ class RMSNorm(Part):
         hand, the norm is not run: a :class:`~gesso_amd.kernels.ops.LazyNorm` goes to the product that
         follows, which norms on the fly.
         """
-        if isinstance(stream.pending, tuple):
+        if isinstance(stream.pending, tuple) or stream.bias is not None:
             stream.flush(self.rt)
         if self.rt.fused and rows is None and stream.pending is None and stream.ssq is not None:
             mine = stream.xs_for is self

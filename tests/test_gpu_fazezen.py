@@ -65,6 +65,14 @@ def test_two_adds_and_two_norms_of_one_row(ops, dtype, H):
             assert float((got.cpu().double() - want).abs().max()) <= tol(dtype, want)
     only, none = ops.add_rmsnorm_pair(res.clone().to(DEV), d1.to(DEV), None, w1.to(DEV), None, 1e-4, dtype)
     assert none is None and only.shape == (5, H)
+    # a vector added to every row on the way (a last product's bias)
+    bias = torch.randn(H, generator=gen(5))
+    r = res.clone().to(DEV)
+    a, _ = ops.add_rmsnorm_pair(r, d1.to(DEV), d2.to(DEV), w1.to(DEV), w2.to(DEV), 1e-4, dtype, bias=bias.to(DEV))
+    x = res.double() + d1.double() + d2.double() + bias.double()
+    assert float((r.cpu().double() - x).abs().max()) <= 1e-6 * float(x.abs().max())
+    want = P.rms(x, 1e-4) * w1.double()
+    assert float((a.cpu().double() - want).abs().max()) <= tol(dtype, want)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -91,7 +99,7 @@ def test_weighted_sum_of_two_results(ops):
 
 
 def scan_case(ops, dtype, H, n, m, lens, rd=0, act=None, scale=1.0, decay=None, seed=0, base=1e3, pos0=None, boost=None,
-              runs_from=0):
+              runs_from=0, segment=0):
     """Rows of q | junk | k | v for sequences of ``lens`` tokens, states in shuffled slots: the kernel's outputs and
     states, and the plain implementation's.  ``pos0``: the first position of each sequence (its state then starts from
     a random one).  ``boost``: ``(sequence, far token, near token)``: that key and that query are made to meet."""
@@ -130,7 +138,7 @@ def scan_case(ops, dtype, H, n, m, lens, rd=0, act=None, scale=1.0, decay=None, 
     if runs_from:
         # sequences of at least that many tokens on the matrix cores, the others token by token, into one result
         out = torch.full((T, H * m), float("nan"), device=DEV)
-        ops.linear_attention_scan(*args, chunks_from=runs_from, out=out, **kw)
+        ops.linear_attention_scan(*args, chunks_from=runs_from, out=out, segment=segment, longest=max(lens), **kw)
         ops.linear_attention_scan(*args, below=runs_from, out=out, **kw)
     else:
         out = ops.linear_attention_scan(*args, **kw)
@@ -179,13 +187,27 @@ def test_fading_state_kernel_on_the_matrix_cores(ops, H, n, m, rd, act, scale, d
     lens, pos0 = [1, 70, 9, 33, 8, 140, 32, 7], [5, 0, 100, 0, 31, 12, 0, 0]
     got, want, state, want_state = scan_case(ops, torch.bfloat16, H, n, m, lens, rd, act, scale, decay=decay and list(decay),
                                              seed=n + m, pos0=pos0, runs_from=8)
-    # activated values enter the products as one bfloat16 term (a projection with its activation); all else as two
-    bound = 4e-3 if act else 1e-4
+    bound = 1e-4
     assert float((got - want).abs().max()) <= bound * max(1.0, float(want.abs().max()))
     for slot, S in want_state.items():
         assert float((state[slot] - S).abs().max()) <= bound * max(1.0, float(S.abs().max()))
     untouched = [s for s in range(state.shape[0]) if s not in want_state]
     assert all(torch.isnan(state[s]).all() for s in untouched)
+
+
+@pytest.mark.parametrize("H,n,m,rd,act,scale,decay,segment", [
+    (2, 64, 64, 0, "silu", 1.0, (0.97, 0.999), 64), (1, 128, 130, 64, None, 0.1, (0.99,), 128), (3, 24, 16, 0, None, 1.0, (1.0, 0.0, 0.9), 32),
+    (2, 32, 64, 32, None, 32 ** -0.5, (0.9, 0.995), 96), (2, 16, 24, 8, None, 0.25, None, 64)])
+def test_fading_state_kernel_with_long_portions_cut_into_segments(ops, H, n, m, rd, act, scale, decay, segment):
+    """Segments side by side, their first states made by a pass between: a last segment of one token, of a whole
+    segment, sequences of one segment only, states that go on from earlier steps."""
+    lens, pos0 = [300, 1, 2 * segment, 40, 2 * segment + 1, 9], [0, 3, 77, 0, 10, 200]
+    got, want, state, want_state = scan_case(ops, torch.bfloat16, H, n, m, lens, rd, act, scale, decay=decay and list(decay),
+                                             seed=n + m + segment, pos0=pos0, runs_from=8, segment=segment)
+    bound = 1e-4
+    assert float((got - want).abs().max()) <= bound * max(1.0, float(want.abs().max()))
+    for slot, S in want_state.items():
+        assert float((state[slot] - S).abs().max()) <= bound * max(1.0, float(S.abs().max()))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
