@@ -52,6 +52,10 @@ struct DecodeRaw {
   const float* cos_t;    // (positions, D / 2)
   const float* sin_t;
   int write_kv;          // 0: another layer owns the cache; the new key is already in it
+  // (read with and without RAW) chunk > 0: the query sees no key before the first position of its own run of `chunk`
+  // positions; sink: one more term exp(0), without a value, in the softmax's denominator
+  int chunk;
+  int sink;
 };
 
 template <int D, int G, int W, int RAW>
@@ -78,7 +82,8 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
   const int pos = positions[seq];
-  const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  if (raw.chunk > 0 && pos - pos % raw.chunk > lo) lo = pos - pos % raw.chunk;
   const int nkeys = pos - lo + 1;
   // this block's share of the keys, in whole tiles of 64
   const int tiles = (nkeys + 63) >> 6;
@@ -398,6 +403,8 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
           L += wl[w][g] * f;
         }
     if (nsplit == 1) {
+      // (a sink's score is 0; the maxima are in base-2 units of the scaled scores)
+      if (raw.sink) L += M > -INFINITY ? __builtin_amdgcn_exp2f(-M) : 1.f;
       out[out_index(seq, (kvh * G + g) * D + j, nh * D, out_tiles)] = f32_to_bf16(o / L);
     } else {
       part_o[(unit * G + g) * D + j] = o;
@@ -415,7 +422,7 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
 #define DEC_MAXSPLIT 64
 __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                               bf16* __restrict__ out, int nsplit, int nh, int nkv, int G, int D,
-                                              int out_tiles) {
+                                              int out_tiles, int sink) {
   __shared__ float sm[DEC_MAXSPLIT][DEC_MAXG], sl[DEC_MAXSPLIT][DEC_MAXG], sf[DEC_MAXSPLIT][DEC_MAXG];
   __shared__ float sinv[DEC_MAXG];
   const int kvh = blockIdx.x, seq = blockIdx.y;
@@ -436,6 +443,7 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
       sf[sp][g] = f;
       L += sl[sp][g] * f;
     }
+    if (sink) L += M > -INFINITY ? __builtin_amdgcn_exp2f(-M) : 1.f;
     sinv[g] = 1.0f / L;
   }
   __syncthreads();
@@ -521,7 +529,8 @@ extern "C" long gs_attention_decode_workspace(int nseq, int nh, int nkv, int d, 
 static int decode_entry(const void* q, int q_stride, void* kcache, void* vcache, const int* positions,
                         const int* block_table, int max_blocks, int page_size, int window, float scale, void* out,
                         int out_tiled, float* workspace, int nseq, int nh, int nkv, int d, int nsplit,
-                        const DecodeRaw* raw, hipStream_t stream) {
+                        const DecodeRaw* raw, hipStream_t stream, int chunk = 0, int sink = 0) {
+  GS_REQUIRE(chunk >= 0, "attention_decode: bad chunk %d", chunk);
   GS_REQUIRE(!out_tiled || (nh * d) % 32 == 0, "attention_decode: tiled rows need a width that is a multiple of 32, not %d", nh * d);
   const int out_tiles = out_tiled ? gs_ceil_div(nseq, 16) : 0;
   GS_REQUIRE(gs_attention_decode_supports(nh, nkv, d), "attention_decode: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
@@ -541,14 +550,19 @@ static int decode_entry(const void* q, int q_stride, void* kcache, void* vcache,
   float* part_o = workspace;
   float* part_ml = workspace + (size_t)nseq * nh * nsplit * d;
   int rc = -1;
-  const DecodeRaw none = {};
+  DecodeRaw none = {};
+  none.chunk = chunk;
+  none.sink = sink ? 1 : 0;
+  DecodeRaw with = raw ? *raw : none;
+  with.chunk = chunk;
+  with.sink = sink ? 1 : 0;
 #define GS_ARGS                                                                                             \
   G, grid, stream, (const bf16*)q, q_stride, (bf16*)kcache, (bf16*)vcache, positions, block_table, max_blocks, \
       page_size, page_magic, window, scale, (bf16*)out, part_o, part_ml, nh, nkv, out_tiles
   if (raw) {
     switch (d) {
-      case 64: rc = launch_decode<64, 1>(GS_ARGS, *raw); break;
-      case 128: rc = launch_decode<128, 1>(GS_ARGS, *raw); break;
+      case 64: rc = launch_decode<64, 1>(GS_ARGS, with); break;
+      case 128: rc = launch_decode<128, 1>(GS_ARGS, with); break;
     }
   } else {
     switch (d) {
@@ -563,7 +577,8 @@ static int decode_entry(const void* q, int q_stride, void* kcache, void* vcache,
   GS_LAUNCH_CHECK("attention_decode");
   if (nsplit > 1) {
     dim3 mgrid(nkv, nseq);
-    attention_decode_merge_kernel<<<mgrid, 256, 0, stream>>>(part_o, part_ml, (bf16*)out, nsplit, nh, nkv, G, d, out_tiles);
+    attention_decode_merge_kernel<<<mgrid, 256, 0, stream>>>(part_o, part_ml, (bf16*)out, nsplit, nh, nkv, G, d, out_tiles,
+                                                             sink ? 1 : 0);
     GS_LAUNCH_CHECK("attention_decode_merge");
   }
   return 0;
@@ -575,6 +590,15 @@ extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcac
                                    int nkv, int d, int nsplit, hipStream_t stream) {
   return decode_entry(q, q_stride, (void*)kcache, (void*)vcache, positions, block_table, max_blocks, page_size, window,
                       scale, out, out_tiled, workspace, nseq, nh, nkv, d, nsplit, nullptr, stream);
+}
+
+// The same with runs of positions and a sink (see DecodeRaw).
+extern "C" int gs_attention_decode_runs(const void* q, int q_stride, const void* kcache, const void* vcache,
+                                        const int* positions, const int* block_table, int max_blocks, int page_size,
+                                        int window, float scale, void* out, int out_tiled, float* workspace, int nseq,
+                                        int nh, int nkv, int d, int nsplit, int chunk, int sink, hipStream_t stream) {
+  return decode_entry(q, q_stride, (void*)kcache, (void*)vcache, positions, block_table, max_blocks, page_size, window,
+                      scale, out, out_tiled, workspace, nseq, nh, nkv, d, nsplit, nullptr, stream, chunk, sink);
 }
 
 // ---- the entry point that allocates nothing (declared and described in no_alloc.h)

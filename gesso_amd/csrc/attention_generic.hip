@@ -114,15 +114,15 @@ extern "C" int gs_attention_generic(const void* q, int q_stride, const void* kca
                                     int max_blocks, int page_size, int window, float scale, void* out, int ntok,
                                     int nh, int nkv, int d, int vd, int chunk, int sink, const float* vcos,
                                     const float* vsin, int interleaved, hipStream_t stream) {
-  GS_REQUIRE(vd > 0 && vd <= GS_ATTN_MAX_D, "attention: value width %d outside 1..%d", vd, GS_ATTN_MAX_D);
-  GS_REQUIRE(chunk >= 0, "attention: bad chunk %d", chunk);
-  GS_REQUIRE((vcos == nullptr) == (vsin == nullptr) && (!vcos || vd % 2 == 0), "attention: value tables come together, for even widths");
   GS_REQUIRE(ntok >= 0 && nh > 0 && nkv > 0 && d > 0, "attention: bad sizes T=%d nh=%d nkv=%d d=%d", ntok, nh, nkv, d);
   GS_REQUIRE(nh % nkv == 0, "attention: %d query heads are no multiple of %d key heads", nh, nkv);
   GS_REQUIRE(d <= GS_ATTN_MAX_D, "attention: head width %d above the kernel's limit %d", d, GS_ATTN_MAX_D);
   GS_REQUIRE(nh <= 65535, "attention: more than 65535 heads");
   GS_REQUIRE(page_size > 0 && max_blocks > 0 && window >= 0, "attention: bad page_size/max_blocks/window");
   GS_REQUIRE(q_stride >= nh * d, "attention: q_stride %d below nh*d %d", q_stride, nh * d);
+  GS_REQUIRE(vd > 0 && vd <= GS_ATTN_MAX_D, "attention: value width %d outside 1..%d", vd, GS_ATTN_MAX_D);
+  GS_REQUIRE(chunk >= 0, "attention: bad chunk %d", chunk);
+  GS_REQUIRE((vcos == nullptr) == (vsin == nullptr) && (!vcos || vd % 2 == 0), "attention: value tables come together, for even widths");
   if (ntok == 0) return 0;
   dim3 grid(ntok, nh);
   if (dtype == GS_F32)

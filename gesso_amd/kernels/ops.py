@@ -909,9 +909,10 @@ def _decode_workspace(device, nseq, nh, nkv, d, nsplit):
 
 
 def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_size, window, scale, nh, nkv, d, nseq,
-                     nsplit: int, out=None):
+                     nsplit: int, out=None, chunk: int = None, sink: bool = False):
     """One query per sequence over its paged keys (bfloat16), keys split over ``nsplit`` blocks per key head.
-    ``out``: a tensor, or True / a :class:`TiledRows` for tiled rows."""
+    ``out``: a tensor, or True / a :class:`TiledRows` for tiled rows.  ``chunk``: the query sees only the keys of its
+    own run of ``chunk`` positions; ``sink``: one more term ``exp(0)`` in the softmax's denominator."""
     _dev(q, kcache, vcache, positions, block_table, out if isinstance(out, torch.Tensor) else None)
     _need(q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
           "attention_decode takes bfloat16")
@@ -924,6 +925,13 @@ def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_s
     ws = _decode_workspace(q.device, nseq, nh, nkv, d, nsplit)
     out, buf, tiled = _rows_out(out, nseq, nh * d, q.device, q.dtype)
     _need(tuple(out.shape) == (nseq, nh * d) and out.dtype == q.dtype, "attention_decode: out has the wrong shape or type")
+    if chunk or sink:
+        _check(lib().gs_attention_decode_runs(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(block_table),
+                                              c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0),
+                                              c_float(scale), _p(buf), c_int(tiled), _p(ws), c_int(nseq), c_int(nh),
+                                              c_int(nkv), c_int(d), c_int(nsplit), c_int(chunk or 0),
+                                              c_int(1 if sink else 0), _stream()))
+        return out
     _check(lib().gs_attention_decode(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(block_table),
                                      c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0), c_float(scale),
                                      _p(buf), c_int(tiled), _p(ws), c_int(nseq), c_int(nh), c_int(nkv), c_int(d),

@@ -213,6 +213,21 @@ class Attention(Part):
         s, rt, ops, vp = self.spec, self.rt, self.rt.ops, self.value_position
         layout = getattr(vp, "layout", "half") if vp is not None else "half"
         nh, nkv, d = s.n_heads, s.n_kv_heads, s.head_dim
+        if (q.dtype == torch.bfloat16 and ctx.all_single and self.value_dim == d and cache.page_size >= 2
+                and q_stride % 8 == 0 and ops.attention_decode_supports(nh, nkv, d)):
+            # single tokens whose values are as wide as their keys: the kernel for single queries, which knows runs and
+            # the sink (its keys reach back to the run's start at most)
+            longest = ctx.max_kv_len if ctx.max_kv_len is not None else cache.block_table.shape[1] * cache.page_size
+            for reach in (s.window, self.chunk):
+                if reach:
+                    longest = min(longest, reach)
+            tiles = max(1, -(-longest // 64))
+            nsplit = max(1, min(tiles // 16, 64, 256 // max(1, ctx.nseq * nkv)))
+            out = ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table, cache.page_size,
+                                       s.window, self.scale, nh, nkv, d, ctx.nseq, nsplit, chunk=self.chunk, sink=self.sink)
+            if vp is not None:
+                ops.turn_heads(out, vp.cos, vp.sin, ctx.positions, nh, d, sign=-1.0, layout=layout)
+            return out
         if (q.dtype == torch.bfloat16 and not ctx.all_single and self.value_dim == d and cache.page_size >= 2
                 and q_stride % 8 == 0 and ops.attention_prefill_supports(nh, nkv, d) and ctx.recording is None):
             # prompt portions whose values are as wide as their keys: the kernel on the matrix cores, which knows runs

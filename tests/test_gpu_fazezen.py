@@ -307,6 +307,12 @@ def attention_case(ops, dtype, nh, nkv, d, vd, rd, chunk, T, page_size, seed, si
                                       chunk=chunk, sink=sink)
             outs.append(ops.turn_heads(o, vcos, vsin, i32(pos[a:b]), nh, vd, sign=-1.0) if turned else o)
             continue
+        if cores:
+            # a single token: the kernel for single queries, its keys in one part and in three
+            o = ops.attention_decode(part, width, kc, vc, i32(pos[a:b]), bt, page_size, None, 0.3, nh, nkv, d, 1, 1 + 2 * (a % 2),
+                                     chunk=chunk, sink=sink)
+            outs.append(ops.turn_heads(o, vcos, vsin, i32(pos[a:b]), nh, vd, sign=-1.0) if turned else o)
+            continue
         outs.append(ops.attention_generic(part, width, kc, vc, i32(pos[a:b]), seq, bt, page_size, None, 0.3, nh, nkv, d, b - a,
                                           vd=vd, chunk=chunk, sink=sink, vcos=vcos, vsin=vsin))
     got = torch.cat(outs).cpu().double()
@@ -351,6 +357,9 @@ def test_attention_within_runs_on_the_matrix_cores(ops, nh, nkv, d, rd, chunk, p
     assert float((got - want).abs().max()) <= tol(torch.bfloat16, want, 2e-5, 2e-2)
     got, want, _ = attention_case(ops, torch.bfloat16, nh, nkv, d, d, rd, chunk, 70, ps, seed=d, sink=False, turned=False, cores=True)
     assert float((got - want).abs().max()) <= tol(torch.bfloat16, want, 2e-5, 2e-2)
+    # the last tokens one by one through the kernel for single queries
+    got, want, _ = attention_case(ops, torch.bfloat16, nh, nkv, d, d, rd, chunk, 150, ps, seed=d + 1, cores=True, single_from=105)
+    assert float((got - want).abs().max()) <= tol(torch.bfloat16, want, 2e-5, 2e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -384,10 +393,12 @@ def test_a_key_that_stands_out_is_found_at_the_edges_of_runs_and_pages_and_far_b
             assert near == seen, (kj, single_from)
         if dtype == torch.bfloat16:
             # the same through the kernel on the matrix cores (keys and values 32 wide)
-            got, want, v = attention_case(ops, dtype, 2, 1, 32, 32, 16, chunk, T, ps, seed=kj, boost=(qi, kj), norm=False, cores=True)
-            assert float((got - want).abs().max()) <= tol(dtype, want, 3e-5, 3e-2), kj
-            alone = P.turn(v[kj:kj + 1, 0], [qi], P.frequencies(32, 1e4), sign=-1.0)[0]
-            assert (float((got[qi, :32] - alone).abs().max()) <= 0.05 * float(alone.abs().max())) == seen, kj
+            for single_from in (None, qi - 2):
+                got, want, v = attention_case(ops, dtype, 2, 1, 32, 32, 16, chunk, T, ps, seed=kj, boost=(qi, kj), norm=False,
+                                              cores=True, single_from=single_from)
+                assert float((got - want).abs().max()) <= tol(dtype, want, 3e-5, 3e-2), (kj, single_from)
+                alone = P.turn(v[kj:kj + 1, 0], [qi], P.frequencies(32, 1e4), sign=-1.0)[0]
+                assert (float((got[qi, :32] - alone).abs().max()) <= 0.05 * float(alone.abs().max())) == seen, (kj, single_from)
 
 
 # ------------------------------------------------------------------ the mixers alone, with their own caches
