@@ -625,7 +625,70 @@ __global__ void add_rmsnorm_pair_kernel(float* __restrict__ res, const TD* __res
   float* x = res + (size_t)r * H;
   const TD* a = d1 ? d1 + (size_t)r * H : nullptr;
   const TD* b = d2 ? d2 + (size_t)r * H : nullptr;
+  TO* o1 = out1 + (size_t)r * H;
+  TO* o2 = out2 ? out2 + (size_t)r * H : nullptr;
   float ss = 0.f;
+  if ((H & 7) == 0 && aligned16(x) && aligned16(o1) && aligned16(w1) && (!o2 || (aligned16(o2) && aligned16(w2))) &&
+      (!a || aligned16(a)) && (!b || aligned16(b)) && (!bias || aligned16(bias))) {
+    // eight values per thread and turn, 16-byte accesses; the row stays in registers between the passes
+    constexpr int MAXV = 4;                       // turns kept in registers: rows up to 8 * 256 * 4 values
+    float keep[MAXV][8];
+    const int turns = (H / 8 + blockDim.x - 1) / blockDim.x;
+    for (int u = 0; u < turns; ++u) {
+      const int j = (u * blockDim.x + threadIdx.x) * 8;
+      float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (j < H) {
+        load8f(x + j, v);
+        float t8[8];
+        if (a) {
+          load8f(a + j, t8);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v[i] += t8[i];
+        }
+        if (b) {
+          load8f(b + j, t8);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v[i] += t8[i];
+        }
+        if (bias) {
+          load8f(bias + j, t8);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v[i] += t8[i];
+        }
+        if (a || b || bias) store8f(x + j, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
+      }
+      if (u < MAXV) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) keep[u][i] = v[i];
+      }
+    }
+    ss = block_sum(ss, red);
+    const float inv = norm_inverse(ss, (float)H, eps);
+    for (int u = 0; u < turns; ++u) {
+      const int j = (u * blockDim.x + threadIdx.x) * 8;
+      if (j >= H) break;
+      float v[8], w8[8], y[8];
+      if (u < MAXV) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = keep[u][i];
+      } else {
+        load8f(x + j, v);                          // (this thread stored it itself)
+      }
+      load8f(w1 + j, w8);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = v[i] * inv * w8[i];
+      store8f(o1 + j, y);
+      if (o2) {
+        load8f(w2 + j, w8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = v[i] * inv * w8[i];
+        store8f(o2 + j, y);
+      }
+    }
+    return;
+  }
   for (int j = threadIdx.x; j < H; j += blockDim.x) {
     float v = x[j];
     if (a) v += to_f32(a[j]);
@@ -636,8 +699,6 @@ __global__ void add_rmsnorm_pair_kernel(float* __restrict__ res, const TD* __res
   }
   ss = block_sum(ss, red);
   const float inv = norm_inverse(ss, (float)H, eps);
-  TO* o1 = out1 + (size_t)r * H;
-  TO* o2 = out2 ? out2 + (size_t)r * H : nullptr;
   for (int j = threadIdx.x; j < H; j += blockDim.x) {
     const float v = x[j] * inv;                 // (this thread wrote x[j] itself)
     o1[j] = from_f32<TO>(v * w1[j]);

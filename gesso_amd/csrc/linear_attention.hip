@@ -150,6 +150,39 @@ __global__ void gated_outnorm_kernel(const float* __restrict__ o, const TI* __re
   const float* row = o + (size_t)t * W;
   const TI* g = gate + (size_t)t * ldg + og;
   TO* dst = out + (size_t)t * W;
+  if (joint && (W & 7) == 0 && W <= 8 * 256 * 4 && aligned16(row) && aligned16(g) && aligned16(dst) && (!w || aligned16(w))) {
+    // eight values a thread and turn, the row in registers between the two passes (rows up to 8192 values)
+    float keep[4][8];
+    float ss = 0.f;
+    const int turns = (W / 8 + blockDim.x - 1) / blockDim.x;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = (u * blockDim.x + threadIdx.x) * 8;
+      if (u < turns && c < W) {
+        load8f(row + c, keep[u]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += keep[u][i] * keep[u][i];
+      }
+    }
+    ss = block_sum(ss, red);
+    const float inv = norm_inverse(ss, (float)W, eps);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = (u * blockDim.x + threadIdx.x) * 8;
+      if (u < turns && c < W) {
+        float z[8], w8[8], y[8];
+        load8f(g + c, z);
+        if (w) load8f(w + c, w8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float sg = 1.0f / (1.0f + expf(-z[i]));
+          y[i] = keep[u][i] * inv * (w ? w8[i] : 1.f) * (gate_act ? z[i] * sg : sg);
+        }
+        store8f(dst + c, y);
+      }
+    }
+    return;
+  }
   if (joint) {
     float ss = 0.f;
     for (int c = threadIdx.x; c < W; c += blockDim.x) ss += row[c] * row[c];
