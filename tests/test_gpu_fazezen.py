@@ -299,7 +299,7 @@ def attention_case(ops, dtype, nh, nkv, d, vd, rd, chunk, T, page_size, seed, si
         seq = torch.zeros(b - a, dtype=torch.int32, device=DEV)
         ops.qknorm_rope_kv(part, dev(qw), dev(kw), 1e-5, cos, sin, rd, i32(pos[a:b]), seq, bt, page_size, kc, vc, nh, nkv, d,
                            vd=vd, vcos=vcos, vsin=vsin)
-        if cores and b - a > 1:
+        if cores is True and b - a > 1:
             # the kernel on the matrix cores, in tiles of 16 queries, and the heads' sums turned back afterwards
             tiles = torch.tensor([[0] * len(range(0, b - a, 16)), list(range(0, b - a, 16)),
                                   [min(16, b - a - r) for r in range(0, b - a, 16)]], dtype=torch.int32, device=DEV)
@@ -307,7 +307,7 @@ def attention_case(ops, dtype, nh, nkv, d, vd, rd, chunk, T, page_size, seed, si
                                       chunk=chunk, sink=sink)
             outs.append(ops.turn_heads(o, vcos, vsin, i32(pos[a:b]), nh, vd, sign=-1.0) if turned else o)
             continue
-        if cores:
+        if cores and b - a == 1:
             # a single token: the kernel for single queries, its keys in one part and in three
             o = ops.attention_decode(part, width, kc, vc, i32(pos[a:b]), bt, page_size, None, 0.3, nh, nkv, d, 1, 1 + 2 * (a % 2),
                                      chunk=chunk, sink=sink)
@@ -359,6 +359,14 @@ def test_attention_within_runs_on_the_matrix_cores(ops, nh, nkv, d, rd, chunk, p
     assert float((got - want).abs().max()) <= tol(torch.bfloat16, want, 2e-5, 2e-2)
     # the last tokens one by one through the kernel for single queries
     got, want, _ = attention_case(ops, torch.bfloat16, nh, nkv, d, d, rd, chunk, 150, ps, seed=d + 1, cores=True, single_from=105)
+    assert float((got - want).abs().max()) <= tol(torch.bfloat16, want, 2e-5, 2e-2)
+
+
+@pytest.mark.parametrize("nh,nkv,d,rd,chunk,ps", [(4, 2, 16, 16, 24, 8), (2, 1, 16, 8, None, 16), (8, 1, 32, 32, 5, 4)])
+def test_single_tokens_through_the_kernel_for_single_queries_at_narrow_heads(ops, nh, nkv, d, rd, chunk, ps):
+    """Heads of 16 (and 32) in bfloat16: the prompt through the general kernel, the last 60 tokens one by one through
+    the kernel for single queries, with runs, the sink and turned values."""
+    got, want, _ = attention_case(ops, torch.bfloat16, nh, nkv, d, d, rd, chunk, 130, ps, seed=7 * d + nh, cores="single", single_from=70)
     assert float((got - want).abs().max()) <= tol(torch.bfloat16, want, 2e-5, 2e-2)
 
 
@@ -600,6 +608,19 @@ def test_replay_four_ways(name, dtype, folders, tmp_path):
         mine = {k.split(".", 1)[1]: v for k, v in got.items() if k.startswith(way + ".")}
         assert {k: len(v) for k, v in mine.items()} == {k: len(v) for k, v in seqs.items()}, way
         plain.check(mine, f"Fazezen {name} {way}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_long_decoding_token_by_token(name, dtype, folders, tmp_path):
+    """A short prompt, then three hundred tokens one by one: states carried and runs begun and ended many times over."""
+    cfg, seed = CONFIGS[name]
+    model_dir = write_tiny(folders, name, torch.float32 if dtype == "float32" else torch.bfloat16)
+    seqs = {"long": random_ids(330, cfg.vocab, 7000 + seed), "other": random_ids(301, cfg.vocab, 7100 + seed)}
+    plain = R.Plain(model_dir, seqs, dtype)
+    got, rc = R.run_trace(model_dir, dtype, str(tmp_path / "out"), R.trace_tail(seqs, tail=300), cfg.vocab)
+    assert rc == 0 and {k: len(v) for k, v in got.items()} == {"long": 330, "other": 301}
+    plain.check(got, f"Fazezen {name}, 300 tokens one by one")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
