@@ -432,8 +432,6 @@ static void lm_launch(dim3 grid, hipStream_t stream, const bf16* x, int ld, int 
                                                                            seg_len);
 }
 
-extern "C" int gs_linear_attention_chunks_max_key() { return 128; }
-
 extern "C" int gs_linear_attention_chunks(const void* x, int ld, int oq, int ok, int ov, int act, const float* cos_t,
                                           const float* sin_t, int rd, int max_position, float key_scale,
                                           const float* decay, float* state, const int* q_start, const int* slots,

@@ -84,7 +84,7 @@ def fazezen_spec(cfg: FazezenConfig) -> ModelSpec:
     # a file may hold the second norm of a layer without a feed-forward; nobody reads it
     return ModelSpec(architecture=ARCHITECTURE, hidden=W, vocab=cfg.vocab, blocks=tuple(blocks),
                      schedule=tuple(LayerCall(i) for i in range(len(blocks))), final_norm=norm, tie_embeddings=True,
-                     max_position=cfg.max_position, names=names, embed_norm=norm)
+                     max_position=cfg.max_position, names=names, embed_norm=norm, ignored_tensors=(".norm2",))
 
 
 register_architecture(ARCHITECTURE, FazezenConfig.from_dict, fazezen_spec, FazezenConfig.to_json)

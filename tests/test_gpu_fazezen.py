@@ -683,6 +683,30 @@ def test_the_command_line_serves_a_fazezen_folder(folders):
     assert json.loads(r.stdout.strip().splitlines()[-1])["ids"] == [want]
 
 
+def test_seventy_requests_at_once_decode_through_the_loop_for_many_rows(folders):
+    """More requests than the weight-streaming products take rows: the recorded loop over the many-row kernels, seventy
+    states and block tables side by side.  Every token chosen is one the plain model ranks near its best at that place,
+    and so is every token the first request gets when it runs alone."""
+    from gesso_amd import Session
+    from noise import supported
+    cfg, _ = CONFIGS["C"]
+    model_dir = write_tiny(folders, "C", torch.bfloat16)
+    pc, pw = P.read_config(model_dir), P.read_weights(model_dir)
+    prompts = [random_ids(3 + (7 * i) % 40, cfg.vocab, 2000 + i) for i in range(70)]
+    session = Session(model_dir, dtype="bfloat16", device=DEV, context_length=128, max_num_seqs=128)
+    try:
+        got = session.generate(prompts, max_new_tokens=12)
+        alone = session.generate([prompts[0]], max_new_tokens=12)[0]
+    finally:
+        session.close()
+    assert [len(g) for g in got] == [len(p) + 12 for p in prompts]
+    for i in (0, 33, 69):
+        lg = P.forward(pc, pw, got[i]).numpy()
+        assert all(supported(lg[j - 1], got[i][j], 0.5) for j in range(len(prompts[i]), len(got[i]))), i
+    lg = P.forward(pc, pw, alone).numpy()
+    assert all(supported(lg[j - 1], alone[j], 0.5) for j in range(len(prompts[0]), len(alone)))
+
+
 def random_fazezen(seed: int):
     """A configuration drawn from a seed: two to four layers of either kind in any order, sizes with and without whole
     tiles, runs shorter and longer than the sequences or none, turns over a part of a head, all of it or none, layers
