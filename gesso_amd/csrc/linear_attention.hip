@@ -107,7 +107,7 @@ extern "C" int gs_linear_attention_scan(const void* x, int dtype, int ld, int oq
                                         const int* slots, const int* positions, float* out, int nseq, int H, int n,
                                         int m, int below, hipStream_t stream) {
   GS_REQUIRE(nseq >= 0 && H > 0 && n > 0 && m > 0, "linear_attention: bad sizes nseq=%d H=%d n=%d m=%d", nseq, H, n, m);
-  GS_REQUIRE(n <= 256, "linear_attention: keys of %d features, the kernel holds up to 256", n);
+  GS_REQUIRE(n <= 512, "linear_attention: keys of %d features, the kernel holds up to 512", n);
   GS_REQUIRE(H <= 65535 && (m + LA_COLS - 1) / LA_COLS <= 65535, "linear_attention: too many heads or value columns");
   GS_REQUIRE(rd >= 0 && rd <= n && rd % 2 == 0, "linear_attention: %d turned features of %d", rd, n);
   GS_REQUIRE(rd == 0 || (cos_t && sin_t && max_position > 0), "linear_attention: rotation without a table");
@@ -124,7 +124,8 @@ extern "C" int gs_linear_attention_scan(const void* x, int dtype, int ld, int oq
   if (n <= 32) LA_RUN(TI, 8);             \
   else if (n <= 64) LA_RUN(TI, 16);       \
   else if (n <= 128) LA_RUN(TI, 32);      \
-  else LA_RUN(TI, 64)
+  else if (n <= 256) LA_RUN(TI, 64);      \
+  else LA_RUN(TI, 128)
   if (dtype == GS_F32) {
     LA_RUN_T(float);
   } else if (dtype == GS_BF16) {

@@ -185,8 +185,10 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
           }
           kv *= key_scale;
           lm_split(qv, qh[e], ql[e]);
-          lm_split(kv, kh[e], kl[e]);
-          lm_split(kv * kdec, KTh[(i + e) * LM_LDT + t], KTl[(i + e) * LM_LDT + t]);
+          if constexpr (MODE != 2) {
+            lm_split(kv, kh[e], kl[e]);
+            lm_split(kv * kdec, KTh[(i + e) * LM_LDT + t], KTl[(i + e) * LM_LDT + t]);
+          }
         }
         auto pack = [](const uint16_t* v) {
           return make_uint4(v[0] | ((uint32_t)v[1] << 16), v[2] | ((uint32_t)v[3] << 16), v[4] | ((uint32_t)v[5] << 16),
@@ -194,11 +196,13 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
         };
         *reinterpret_cast<uint4*>(Qh + t * LDQ + i) = pack(qh);
         *reinterpret_cast<uint4*>(Ql + t * LDQ + i) = pack(ql);
-        *reinterpret_cast<uint4*>(Kh + t * LDQ + i) = pack(kh);
-        *reinterpret_cast<uint4*>(Kl + t * LDQ + i) = pack(kl);
+        if constexpr (MODE != 2) {     // (the pass that adds a first state's term needs the queries alone)
+          *reinterpret_cast<uint4*>(Kh + t * LDQ + i) = pack(kh);
+          *reinterpret_cast<uint4*>(Kl + t * LDQ + i) = pack(kl);
+        }
       }
 #pragma unroll
-      for (int u = 0; u < UV; ++u) {
+      for (int u = 0; u < (MODE == 2 ? 0 : UV); ++u) {
         const int piece = tid + 256 * u, t = piece % LM_C, c = (piece / LM_C) * 8;
         float v8[8];
         eight(rv[u], v8);
@@ -277,9 +281,10 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
       continue;
     }
     // scores, transposed: rows s, columns t
-    lm_f32x16_t at;
+    // (two accumulators in turn: a product that waits for the one before it idles the pipe for its whole latency)
+    lm_f32x16_t at, at2;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) at[e] = 0.f;
+    for (int e = 0; e < 16; ++e) at[e] = at2[e] = 0.f;
     const int ro = l32 * LDQ + half * 8;
 #pragma unroll
     for (int ks = 0; ks < NP / 16; ++ks) {
@@ -288,9 +293,11 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
       const lm_bf16x8_t qh8 = *reinterpret_cast<const lm_bf16x8_t*>(Qh + ro + ks * 16);
       const lm_bf16x8_t ql8 = *reinterpret_cast<const lm_bf16x8_t*>(Ql + ro + ks * 16);
       at = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh8, qh8, at, 0, 0, 0);
-      at = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh8, ql8, at, 0, 0, 0);
-      at = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kl8, qh8, at, 0, 0, 0);
+      at2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh8, ql8, at2, 0, 0, 0);
+      at2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kl8, qh8, at2, 0, 0, 0);
     }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) at[e] += at2[e];
     // this lane: query t = l32, keys s(e); the causal rule and the decay between the two; as operands of the next product
     lm_bf16x8_t ah[2], al[2];
 #pragma unroll
@@ -302,9 +309,9 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
       al[e / 8][e % 8] = __builtin_bit_cast(__bf16, f32_to_bf16(a - to_f32(hi)).x);
     }
     // what the state before the run gives: rows t, columns j, then each row times d^(t+1)
-    lm_f32x16_t o;
+    lm_f32x16_t o, ob;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) o[e] = 0.f;
+    for (int e = 0; e < 16; ++e) o[e] = ob[e] = 0.f;
     const int so = (jw + l32) * LDQ + half * 8;
 #pragma unroll
     for (int ks = 0; ks < NP / 16; ++ks) {
@@ -313,11 +320,11 @@ __global__ __launch_bounds__(256) void linear_attention_chunk_kernel(
       const lm_bf16x8_t sh8 = *reinterpret_cast<const lm_bf16x8_t*>(STh + so + ks * 16);
       const lm_bf16x8_t sl8 = *reinterpret_cast<const lm_bf16x8_t*>(STl + so + ks * 16);
       o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qh8, sh8, o, 0, 0, 0);
-      o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qh8, sl8, o, 0, 0, 0);
-      o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ql8, sh8, o, 0, 0, 0);
+      ob = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qh8, sl8, ob, 0, 0, 0);
+      ob = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ql8, sh8, ob, 0, 0, 0);
     }
 #pragma unroll
-    for (int e = 0; e < 16; ++e) o[e] *= pw[8 * (e / 4) + 4 * half + e % 4 + 1];
+    for (int e = 0; e < 16; ++e) o[e] = (o[e] + ob[e]) * pw[8 * (e / 4) + 4 * half + e % 4 + 1];
     // what the run's own tokens give
     const int vo = (jw + l32) * LM_LDT;
 #pragma unroll

@@ -384,7 +384,7 @@ def attention_generic(q, q_stride, kcache, vcache, positions, seq_of_token, bloc
 _ACTS = {None: 0, "none": 0, "silu": 1}
 _GATES = {"sigmoid": 0, "silu": 1}
 GATED_ACTS = {"silu": 0, "gelu_tanh": 1}
-LINEAR_ATTENTION_MAX_KEY = 256
+LINEAR_ATTENTION_MAX_KEY = 512
 LINEAR_ATTENTION_CHUNKS_MAX_KEY = 128
 
 

@@ -167,7 +167,8 @@ def scan_case(ops, dtype, H, n, m, lens, rd=0, act=None, scale=1.0, decay=None, 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,n,m,rd,act,scale", [(3, 24, 16, 0, "silu", 1.0), (2, 16, 24, 8, None, 0.25), (1, 40, 48, 40, None, 0.5),
                                                 (2, 64, 64, 0, "silu", 1.0), (1, 128, 130, 64, None, 0.1), (5, 6, 10, 2, None, 1.0),
-                                                (1, 200, 70, 0, None, 0.3), (2, 32, 64, 32, None, 32 ** -0.5)])
+                                                (1, 200, 70, 0, None, 0.3), (2, 32, 64, 32, None, 32 ** -0.5), (1, 300, 40, 300, None, 0.05),
+                                                (1, 512, 8, 0, "silu", 0.1)])
 def test_fading_state_kernel_over_unequal_sequences(ops, dtype, H, n, m, rd, act, scale):
     got, want, state, want_state = scan_case(ops, dtype, H, n, m, [1, 19, 2, 33], rd, act, scale, seed=n + m)
     assert float((got - want).abs().max()) <= 5e-5 * max(1.0, float(want.abs().max()))     # float32 arithmetic in both types
